@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from ..kernels import runtime as rt
-from ..parts.base import KvNeed, StateNeed
+from ..parts.base import KvNeed, StateNeed, flat_needs
 from .pages import PAGE_TOKENS, CacheError, pages_for
 
 
@@ -112,23 +112,14 @@ class SequenceCache:
         self._layer_index = {}
         self._state = {}
         self._h = None
+        self._composite = {}              # cache layer -> the keys of its parts, for a mixer that holds several things
         for i, need in enumerate(needs):
-            if isinstance(need, KvNeed):
-                for gi, g in enumerate(self.groups):
-                    if g.need == need:
-                        break
-                else:
-                    gi = len(self.groups)
-                    self.groups.append(_Group(need, []))
-                self._layer_group[i] = gi
-                self._layer_index[i] = len(self.groups[gi].layers)
-                self.groups[gi].layers.append(i)
-            elif isinstance(need, StateNeed):
-                # one row more than slots: the padding rows of a captured step keep their state there
-                self._state[i] = torch.zeros((self.max_slots + 1,) + tuple(need.shape), dtype=need.dtype,
-                                             device=self.device)
-            elif need is not None:
-                raise CacheError(f"cache layer {i}: unknown need {need!r}")
+            if isinstance(need, (tuple, list)):
+                self._composite[i] = [(i, j) for j in range(len(need))]
+                for key, part in zip(self._composite[i], flat_needs(need)):
+                    self._register(key, part)
+            else:
+                self._register(i, need)
         if rt.lib().syn_rt_page_tokens() != PAGE_TOKENS:
             raise RuntimeError("the runtime library was built for another page size")
         windows = [-1 if g.need.window is None else int(g.need.window) for g in self.groups]
@@ -136,7 +127,8 @@ class SequenceCache:
             g.n_pages = self.n_pages
             if g.need.window is not None and max_step_tokens is not None:
                 # at most window + step tokens of a sequence are held at once, and they may begin anywhere in a page
-                g.n_pages = min(self.n_pages, self.max_slots * (pages_for(int(g.need.window) + int(max_step_tokens)) + 1))
+                g.n_pages = min(self.n_pages, self.max_slots * (pages_for(int(g.need.window) + int(max_step_tokens)) + 1
+                                                                + pages_for(int(g.need.keep_first))))
         self._h = rt.lib().syn_cache_new(len(self.groups), rt.longs(windows), self.n_pages,
                                          rt.ints([g.n_pages for g in self.groups]), self.max_slots,
                                          -1 if max_positions is None else int(max_positions))
@@ -144,11 +136,33 @@ class SequenceCache:
             raise CacheError(rt.last_error())
         for gi, g in enumerate(self.groups):
             n, nd = len(g.layers), g.need
+            if nd.window is not None and nd.keep_first:
+                rt.check(rt.lib().syn_cache_set_keep_first(self._h, gi, int(nd.keep_first)))
             g.pool = _GroupPool(self, gi, g.n_pages)
             # zeros: what a kernel may touch beyond a sequence's end is at least a number
             g.spare_page = g.n_pages
             g.k = torch.zeros((n, g.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
-            g.v = torch.zeros((n, g.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
+            g.v = torch.zeros((n, g.n_pages + 1, nd.kv_heads, nd.v_dim or nd.head_dim, PAGE_TOKENS), dtype=dtype,
+                              device=self.device)
+
+    def _register(self, key, need) -> None:
+        """One simple need of a cache layer (key: the layer, or (layer, part) inside a tuple of needs)."""
+        if isinstance(need, KvNeed):
+            for gi, g in enumerate(self.groups):
+                if g.need == need:
+                    break
+            else:
+                gi = len(self.groups)
+                self.groups.append(_Group(need, []))
+            self._layer_group[key] = gi
+            self._layer_index[key] = len(self.groups[gi].layers)
+            self.groups[gi].layers.append(key)
+        elif isinstance(need, StateNeed):
+            # one row more than slots: the padding rows of a captured step keep their state there
+            self._state[key] = torch.zeros((self.max_slots + 1,) + tuple(need.shape), dtype=need.dtype,
+                                           device=self.device)
+        elif need is not None:
+            raise CacheError(f"cache layer {key}: unknown need {need!r}")
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -205,7 +219,7 @@ class SequenceCache:
         for g in self.groups:
             n = pages_for(total_tokens)
             if g.need.window is not None:
-                n = min(n, pages_for(int(g.need.window) + int(longest_step)) + 1)
+                n = min(n, pages_for(int(g.need.window) + int(longest_step)) + 1 + pages_for(int(g.need.keep_first)))
             out.append(n)
         return out
 
@@ -270,7 +284,9 @@ class SequenceCache:
         rt.check(rt.lib().syn_cache_page_table(self._h, gi, rt.ints(sids), len(sids), w, out.ctypes.data))
         return out
 
-    def layer_view(self, i: int):
+    def layer_view(self, i):
+        if i in self._composite:
+            return tuple(self.layer_view(key) for key in self._composite[i])
         if i in self._layer_group:
             gi = self._layer_group[i]
             g, li = self.groups[gi], self._layer_index[i]
@@ -286,4 +302,5 @@ class SequenceCache:
 
     def bytes_per_token(self) -> int:
         el = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(2 * len(g.layers) * g.need.kv_heads * g.need.head_dim * el for g in self.groups)
+        return sum(len(g.layers) * g.need.kv_heads * (g.need.head_dim + (g.need.v_dim or g.need.head_dim)) * el
+                   for g in self.groups)

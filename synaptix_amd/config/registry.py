@@ -36,8 +36,8 @@ def known_architectures() -> list:
 
 
 def resolve_architecture(config: dict) -> Architecture:
-    """`architectures[0]` decides; `model_type` is the fallback when it is absent."""
-    names = config.get("architectures") or []
+    """`architectures[0]` (or a single `architecture`) decides; `model_type` is the fallback when it is absent."""
+    names = config.get("architectures") or config.get("architecture") or []
     if isinstance(names, str):
         names = [names]
     for n in names:

@@ -109,9 +109,12 @@ __device__ __forceinline__ float load_gain(const void* w, int is_f32, int i, flo
 // of the 32-bit path).  `act` is a code that the host checks against SYN_ACT_COUNT before any launch;
 // another activation is another case here and another name in the host's table.
 #define SYN_ACT_SILU 0
-#define SYN_ACT_COUNT 1
+#define SYN_ACT_GELU_TANH 1
+#define SYN_ACT_COUNT 2
 __device__ __forceinline__ float gate_activation(int act, float g) {
   switch (act) {
+    case SYN_ACT_GELU_TANH:  // 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+      return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     default:  // SYN_ACT_SILU: z / (1 + e^-z)
       return g / (1.f + expf(-g));
   }

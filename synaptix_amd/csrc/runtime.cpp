@@ -93,6 +93,7 @@ struct Slot {
 struct Cache {
   std::vector<PagePool> pools;   // one for each group
   std::vector<long> windows;     // keys a query sees, or -1 for all of them
+  std::vector<long> keep_first;  // with a window: the first keys of a sequence that every later query still sees
   int n_pages, max_slots;
   long max_positions;            // -1: no limit
   std::vector<Slot> slots;
@@ -202,10 +203,18 @@ RT_API void* syn_cache_new(int n_groups, const long* windows, int n_pages, const
   for (int g = 0; g < n_groups; ++g) {
     c->pools.emplace_back(group_pages ? group_pages[g] : n_pages);
     c->windows.push_back(windows[g]);
+    c->keep_first.push_back(0);
   }
   c->slots.resize(max_slots);
   for (int s = max_slots - 1; s >= 0; --s) c->free_slots.push_back(s);
   return c;
+}
+// a group with a window never gives back the pages that hold a sequence's first n keys
+RT_API int syn_cache_set_keep_first(void* h, int group, long n) {
+  Cache* c = (Cache*)h;
+  if (group < 0 || group >= (int)c->pools.size() || n < 0) return fail(MISUSE, "group %d keeps %ld first keys", group, n);
+  c->keep_first[group] = n;
+  return OK;
 }
 RT_API void syn_cache_delete(void* h) { delete (Cache*)h; }
 RT_API int syn_cache_free_slots(void* h) { return (int)((Cache*)h)->free_slots.size(); }
@@ -319,7 +328,7 @@ RT_API int syn_cache_commit(void* h, int sid, long n_new) {
     // the next query sits at position `length`; it sees keys > length - w
     const long first_needed = std::max(0L, s->length - w + 1) / PAGE_TOKENS;
     std::vector<int>& pages = s->pages[g];
-    for (long i = 0; i < first_needed && i < (long)pages.size(); ++i)
+    for (long i = pages_for(c->keep_first[g]); i < first_needed && i < (long)pages.size(); ++i)
       if (pages[i] >= 0) {
         const int rc = c->pools[g].give_back(&pages[i], 1);
         if (rc) return rc;

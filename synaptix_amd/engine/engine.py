@@ -58,11 +58,11 @@ class Engine:
         self._host = None
         self._dev = None
         self._runners = {}
-        from ..parts.base import StateNeed
+        from ..parts.base import StateNeed, flat_needs
         # steps are replayed from graphs only if every part says of itself that it only launches kernels and
         # finds its sequences through arrays on the device (Part.capturable).  A step is run before it is
         # captured; where sequences have running states the runner puts them back after each such run.
-        self.has_states = any(isinstance(n, StateNeed) for n in model.cache_needs())
+        self.has_states = any(isinstance(n, StateNeed) for need in model.cache_needs() for n in flat_needs(need))
         self.graph_ok = bool(getattr(model, "capturable", lambda: False)())
         self.prompt_graphs = True        # short prompt steps are replayed from graphs (see _prompt_runner)
 

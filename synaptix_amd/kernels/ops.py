@@ -139,7 +139,7 @@ def _is_f32(t):
 
 
 # The activations of a gated feed-forward that the kernels apply (codes of gate_activation in csrc/common.h).
-ACTIVATIONS = {"silu": 0, "swish": 0}
+ACTIVATIONS = {"silu": 0, "swish": 0, "gelu_tanh": 1}
 
 
 def activation_code(name) -> int:
@@ -699,6 +699,217 @@ def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out,
           ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0,
           *_score_terms("attention_decode_fused", slopes, softcap, nh),
           *_decode_work("attention_decode_fused", counters, items, B, n_splits, nh, nkv), _stream())
+
+
+# ----------------------------------------------------------------------------- residual streams, dynamic tanh
+
+ROWNORM_NONE, ROWNORM_DYT = 0, 1
+STREAMS_MAX = 16
+
+
+def _streams(X, name):
+    """X as [N, S, W]: a plain residual [N, W] counts as one stream."""
+    _need(X, name, _F32)
+    if X.dim() == 2:
+        return X.shape[0], 1, X.shape[1]
+    if X.dim() != 3 or not (1 <= X.shape[1] <= STREAMS_MAX):
+        raise KernelError(f"{name}: shape {list(X.shape)}, expected [N, W] or [N, S, W] with up to {STREAMS_MAX} streams")
+    return tuple(X.shape)
+
+
+def streams_read_norm(X, in_w, out, dyt=None, rows=None, delta=None):
+    """out[i] = norm(sum_s in_w[s] X[row, s] (+ delta[row])), row = rows[i] or i.  X [N, S, W] float (or [N, W]);
+    in_w float [S] or None (every weight 1: the sum of the streams); dyt = (alpha [1], gain [W], shift [W]) float:
+    tanh(alpha u) gain + shift, None: u itself; delta [N, W] or partial sums [P, N, W] float, with one stream only
+    (without rows it is added into X as well); out [n, W] bf16 or float."""
+    N, S, W = _streams(X, "streams_read_norm.X")
+    if in_w is not None:
+        _need(in_w, "streams_read_norm.in_w", _F32, (S,))
+    n_out = N
+    if rows is not None:
+        _need(rows, "streams_read_norm.rows", _I32, (None,))
+        n_out = rows.shape[0]
+    n_parts = 0
+    if delta is not None:
+        if S != 1:
+            raise KernelError("streams_read_norm: a delta comes with one stream")
+        n_parts = delta.shape[0] if delta.dim() == 3 else 1
+        _need(delta, "streams_read_norm.delta", _F32, (n_parts, N, W) if delta.dim() == 3 else (N, W))
+    alpha = gain = shift = None
+    if dyt is not None:
+        alpha, gain, shift = dyt
+        _need(alpha, "streams_read_norm.alpha", _F32)
+        _need(gain, "streams_read_norm.gain", _F32, (W,))
+        _need(shift, "streams_read_norm.shift", _F32, (W,))
+        if alpha.numel() != 1:
+            raise KernelError("streams_read_norm: alpha is one number")
+    _need(out, "streams_read_norm.out", (_BF16, _F32), (n_out, W))
+    _call(load_library("core"), "syn_streams_read_norm", _ptr(X), _ptr(delta), n_parts, N, _ptr(rows), n_out, _ptr(in_w),
+          S, W, ROWNORM_NONE if dyt is None else ROWNORM_DYT, _ptr(alpha), _ptr(gain), _ptr(shift), _ptr(out),
+          _is_f32(out), _stream())
+
+
+def streams_update(X, mix, out_w, terms):
+    """X[n, t] = sum_s mix[s, t] X[n, s] + out_w[t] y[n] in place, all streams from the old ones;
+    y = sum over `terms` of scale * (sum of the term's partial sums + bias).  terms: one or two (tensor [N, W] or
+    [P, N, W] float, scale, bias [W] float or None)."""
+    N, S, W = _streams(X, "streams_update.X")
+    _need(mix, "streams_update.mix", _F32, (S, S))
+    _need(out_w, "streams_update.out_w", _F32, (S,))
+    if not (1 <= len(terms) <= 2):
+        raise KernelError(f"streams_update: {len(terms)} terms (one or two)")
+    args = []
+    for y, scale, bias in list(terms) + [(None, 0.0, None)] * (2 - len(terms)):
+        parts = 0
+        if y is not None:
+            parts = y.shape[0] if y.dim() == 3 else 1
+            _need(y, "streams_update.y", _F32, (parts, N, W) if y.dim() == 3 else (N, W))
+            if bias is not None:
+                _need(bias, "streams_update.bias", _F32, (W,))
+        args += [_ptr(y), parts, ctypes.c_float(scale), _ptr(bias)]
+    _call(load_library("core"), "syn_streams_update", _ptr(X), N, S, W, _ptr(mix), _ptr(out_w), *args, _stream())
+
+
+def streams_start(x, X):
+    """X[n, s] = x[n] for every stream: x [N, W] float, X [N, S, W] float."""
+    _need(x, "streams_start.x", _F32, (None, None))
+    N, W = x.shape
+    _need(X, "streams_start.X", _F32, (N, None, W))
+    _call(load_library("core"), "syn_streams_start", _ptr(x), _ptr(X), N, X.shape[1], W, _stream())
+
+
+# ----------------------------------------------------------------------------- attention with terms, a kept window, a sink
+
+WINDOW_ATTENTION_MAX_DIM = 256
+
+
+def _check_window_pages(k_pages, v_pages, dtype, nkv, dim, vdim, name):
+    _need(k_pages, name + ".k_pages", dtype, (None, nkv, PAGE_TOKENS, dim))
+    _need(v_pages, name + ".v_pages", dtype, (k_pages.shape[0], nkv, vdim, PAGE_TOKENS))
+
+
+def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
+                  n_heads, n_kv_heads, dim, vdim, write_kv=True):
+    """proj [N, width] float: the fused projection [q | k | v | ...]; bias float [>= q, k, v columns] or None.  q and k
+    heads get their bias and (with gains, float [dim]) an RMSNorm over the head; q goes to q_out [N, nh * dim], k and v
+    (with its bias) into the pages of sequence tok_seq[n] at position tok_pos[n]."""
+    nh, nkv = n_heads, n_kv_heads
+    _need(proj, "window_intake.proj", _F32, (None, None))
+    N, width = proj.shape
+    used = (nh + nkv) * dim + nkv * vdim
+    if width < used:
+        raise KernelError(f"window_intake: rows of {width} values do not hold q, k and v ({used})")
+    if bias is not None:
+        _need(bias, "window_intake.bias", _F32, (None,))
+        if bias.shape[0] < used:
+            raise KernelError(f"window_intake: a bias of {bias.shape[0]} values for {used} columns")
+    _need(q_out, "window_intake.q_out", (_BF16, _F32), (N, nh * dim))
+    _check_window_pages(k_pages, v_pages, q_out.dtype, nkv, dim, vdim, "window_intake")
+    _need(page_table, "window_intake.page_table", _I32, (None, None))
+    _need(tok_seq, "window_intake.tok_seq", _I32, (N,))
+    _need(tok_pos, "window_intake.tok_pos", _I32, (N,))
+    if (q_gain is None) != (k_gain is None):
+        raise KernelError("window_intake: q and k gains come together")
+    if q_gain is not None:
+        _need(q_gain, "window_intake.q_gain", _F32, (dim,))
+        _need(k_gain, "window_intake.k_gain", _F32, (dim,))
+    _call(load_library("core"), "syn_window_intake", _ptr(proj), width, _ptr(bias), _ptr(q_out), _ptr(k_pages),
+          _ptr(v_pages), _is_f32(q_out), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos),
+          _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), N, nh, nkv, dim, vdim, 1 if write_kv else 0, _stream())
+
+
+def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, n_kv_heads, dim, vdim,
+                     window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None, softcap=0.0, gate=None,
+                     gate_bias=None):
+    """Attention of every token (prompts and single tokens alike) whose query is q [N, nh * dim] over the pages
+    (which already hold the tokens): score = scale q.k [soft cap] - slopes[h] (i - j) - r1[h] ln(1 + r2[h] (i - j))
+    with log_bias = (r1, r2) float [nh]; key j is seen by i iff j <= i and (no window or i - j < window or
+    j < keep_first); sink_one: one more in the softmax's denominator; gate: a float view [N, >= nh * vdim] with row
+    stride gate.stride(0) whose sigmoid multiplies the result; out [N, nh * vdim] in q's type."""
+    nh, nkv = n_heads, n_kv_heads
+    _need(q, "window_attention.q", (_BF16, _F32), (None, nh * dim))
+    N = q.shape[0]
+    _check_window_pages(k_pages, v_pages, q.dtype, nkv, dim, vdim, "window_attention")
+    _need(page_table, "window_attention.page_table", _I32, (None, None))
+    _need(tok_seq, "window_attention.tok_seq", _I32, (N,))
+    _need(tok_pos, "window_attention.tok_pos", _I32, (N,))
+    _need(out, "window_attention.out", q.dtype, (N, nh * vdim))
+    if max(dim, vdim) > WINDOW_ATTENTION_MAX_DIM:
+        raise KernelError(f"window_attention: head sizes {dim}, {vdim} exceed {WINDOW_ATTENTION_MAX_DIM}")
+    r1 = r2 = None
+    if log_bias is not None:
+        r1, r2 = log_bias
+        _need(r1, "window_attention.r1", _F32, (nh,))
+        _need(r2, "window_attention.r2", _F32, (nh,))
+    if slopes is not None:
+        _need(slopes, "window_attention.slopes", _F32, (nh,))
+    gate_stride = 0
+    if gate is not None:
+        gate_stride = _float_rows_view(gate, "window_attention.gate", N, nh * vdim)
+        if gate_bias is not None:
+            _need(gate_bias, "window_attention.gate_bias", _F32, (nh * vdim,))
+    _call(load_library("core"), "syn_window_attention", _ptr(q), _ptr(k_pages), _ptr(v_pages), _is_f32(q),
+          _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(gate), gate_stride,
+          _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), N, nh, nkv, dim, vdim,
+          _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
+          1 if sink_one else 0, _stream())
+
+
+def _float_rows_view(t, name, n_rows, n_cols):
+    """A float tensor [n_rows, >= n_cols] whose rows may be pieces of longer rows (columns of a fused projection):
+    returns the row stride in elements."""
+    if not isinstance(t, torch.Tensor) or t.dtype != _F32 or not t.is_cuda or t.dim() != 2:
+        raise KernelError(f"{name}: expected a float matrix on the GPU")
+    if t.shape[0] != n_rows or t.shape[1] < n_cols or t.stride(1) != 1 or t.stride(0) < t.shape[1]:
+        raise KernelError(f"{name}: shape {list(t.shape)} with strides {list(t.stride())}, expected [{n_rows}, >= {n_cols}] rows")
+    return t.stride(0)
+
+
+# ----------------------------------------------------------------------------- matrix memory
+
+MATRIX_MEMORY_MAX_DIM = 256
+
+
+def matrix_memory_state_size(dim, vdim) -> int:
+    """Floats of a (slot, head)'s state: S [dim, vdim] by rows, n [dim], m."""
+    return dim * vdim + dim + 1
+
+
+def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+    """The cell of csrc/matrix_memory.hip over the new tokens of every sequence of the step, in order, from and into
+    state [rows, H, dim * vdim + dim + 1] float (row = seq_slot[b]; a negative slot takes the last row).
+    proj [N, width] float: [q | k | v | gate | i | f] of the fused projection; out [N, H * vdim] float."""
+    H = n_heads
+    _need(proj, "matrix_memory_scan.proj", _F32, (None, None))
+    N, width = proj.shape
+    if width < 2 * H * dim + 2 * H * vdim + 2 * H:
+        raise KernelError(f"matrix_memory_scan: rows of {width} values are too short")
+    if dim > MATRIX_MEMORY_MAX_DIM:
+        raise KernelError(f"matrix_memory_scan: keys of {dim} values (at most {MATRIX_MEMORY_MAX_DIM})")
+    for name, t in (("i_bias", i_bias), ("f_bias", f_bias)):
+        if t is not None:
+            _need(t, f"matrix_memory_scan.{name}", _F32, (H,))
+    _need(state, "matrix_memory_scan.state", _F32, (None, H, matrix_memory_state_size(dim, vdim)))
+    _need(seq_start, "matrix_memory_scan.seq_start", _I32, (None,))
+    B = seq_start.shape[0] - 1
+    _need(seq_slot, "matrix_memory_scan.seq_slot", _I32, (B,))
+    _need(out, "matrix_memory_scan.out", _F32, (N, H * vdim))
+    _call(load_library("core"), "syn_matrix_memory_scan", _ptr(proj), width, _ptr(i_bias), _ptr(f_bias),
+          ctypes.c_float(float(gate_cap or 0.0)), ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(seq_start),
+          _ptr(seq_slot), B, _ptr(out), H, dim, vdim, _stream())
+
+
+def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim):
+    """out[n, h] = o[n, h] / rms(o[n, h]) * gain[h] * sigmoid(gate[n, h]): o [N, H * vdim] float, gain float [H * vdim]
+    or None, gate a float view [N, >= H * vdim] (see _float_rows_view) or None, out [N, H * vdim] bf16 or float."""
+    _need(o, "head_norm_gate.o", _F32, (None, n_heads * vdim))
+    N = o.shape[0]
+    if gain is not None:
+        _need(gain, "head_norm_gate.gain", _F32, (n_heads * vdim,))
+    stride = _float_rows_view(gate, "head_norm_gate.gate", N, n_heads * vdim) if gate is not None else 0
+    _need(out, "head_norm_gate.out", (_BF16, _F32), (N, n_heads * vdim))
+    _call(load_library("core"), "syn_head_norm_gate", _ptr(o), _ptr(gain), ctypes.c_float(eps), _ptr(gate), stride,
+          _ptr(out), _is_f32(out), N, n_heads, vdim, _stream())
 
 
 # ----------------------------------------------------------------------------- sampling

@@ -1,4 +1,5 @@
 from .decoder import DecoderModel, LayerRun, TokenEmbedding, OutputHead
 from .qwen3 import build_qwen3
+from .bizipel import build_bizipel
 
-__all__ = ["DecoderModel", "LayerRun", "TokenEmbedding", "OutputHead", "build_qwen3"]
+__all__ = ["DecoderModel", "LayerRun", "TokenEmbedding", "OutputHead", "build_qwen3", "build_bizipel"]

@@ -73,8 +73,13 @@ class OutputHead(Part):
 
 
 class DecoderModel:
-    def __init__(self, config, embedding: TokenEmbedding, blocks: list, schedule: list, final_norm, head: OutputHead):
+    def __init__(self, config, embedding: TokenEmbedding, blocks: list, schedule: list, final_norm, head: OutputHead,
+                 streams: int | None = None):
+        """streams: the residual runs in this many copies [N, streams, hidden] that all start as the embedding
+        (blocks that read and write them: parts.HyperConnectionBlock; the final norm gets their sum); None: one
+        plain residual [N, hidden]."""
         self.config = config
+        self.streams = streams
         self.embedding, self.blocks, self.schedule = embedding, list(blocks), list(schedule)
         self.final_norm, self.head = final_norm, head
         self.vocab, self.hidden = embedding.vocab, embedding.hidden
@@ -140,6 +145,10 @@ class DecoderModel:
         """tokens [N] int32 and want_rows [n] int32 (or None) on the device; returns logits [n, vocab] float."""
         with ops.stream_scope():     # one stream for the whole pass, asked for once
             resid = self.embedding.forward(tokens)
+            if self.streams is not None:
+                x0, resid = resid, torch.empty((tokens.shape[0], self.streams, self.hidden), dtype=torch.float32,
+                                               device=tokens.device)
+                ops.streams_start(x0, resid)
             pending = None
             for run, owner in zip(self.schedule, self._owner):
                 block = self.blocks[run.block]

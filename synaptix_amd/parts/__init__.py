@@ -1,11 +1,14 @@
-from .base import Part, KvNeed, StateNeed
-from .norm import RmsNorm
-from .position import Position, NoPosition, RotaryHalfSplit
-from .mixer import Mixer, GqaAttention
+from .base import Part, KvNeed, StateNeed, flat_needs
+from .norm import RmsNorm, DynamicTanh
+from .position import Position, NoPosition, RotaryHalfSplit, LogDistanceBias
+from .mixer import Mixer, GqaAttention, GatedWindowAttention, ParallelMixers
+from .memory import MatrixMemory
 from .feedforward import FeedForward, GatedMlp
-from .block import Block, PreNormBlock
-from .linear import (Matrix, linear, linear_for_sum, deferred_product, DeferredProduct, ScaledRows,
+from .block import Block, PreNormBlock, HyperConnectionBlock
+from .linear import (Matrix, linear, linear_for_sum, deferred_product, DeferredProduct, ScaledRows, WeightedDeltas,
                      as_rows, as_delta)
 
-__all__ = ["Part", "KvNeed", "StateNeed", "RmsNorm", "Position", "NoPosition", "RotaryHalfSplit", "Mixer",
-           "GqaAttention", "FeedForward", "GatedMlp", "Block", "PreNormBlock", "linear", "Matrix"]
+__all__ = ["Part", "KvNeed", "StateNeed", "flat_needs", "RmsNorm", "DynamicTanh", "Position", "NoPosition",
+           "RotaryHalfSplit", "LogDistanceBias", "Mixer", "GqaAttention", "GatedWindowAttention", "ParallelMixers",
+           "MatrixMemory", "FeedForward", "GatedMlp", "Block", "PreNormBlock", "HyperConnectionBlock", "linear", "Matrix",
+           "WeightedDeltas"]

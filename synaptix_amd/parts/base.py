@@ -42,6 +42,16 @@ class KvNeed:
     kv_heads: int
     head_dim: int
     window: Optional[int] = None      # None: all keys
+    v_dim: Optional[int] = None       # size of a value where it differs from the keys' (None: head_dim)
+    keep_first: int = 0               # with a window: the first keys of a sequence that stay visible for good
+
+
+def flat_needs(need) -> tuple:
+    """A mixer's need as a tuple of simple needs: a mixer that holds several things (keys and values for one half,
+    a running state for the other) returns a tuple, which its cache view then mirrors."""
+    if need is None:
+        return ()
+    return tuple(need) if isinstance(need, (tuple, list)) else (need,)
 
 
 @dataclass(frozen=True)

@@ -62,3 +62,83 @@ class PreNormBlock(Block):
         a = self.mixer.forward(h if self.mixer.takes_scaled_rows else as_rows(h), ctx, cache, owner)
         h2 = self.norm2.add_apply(resid, _norm_input(self.norm2, a), ctx.act_dtype)
         return self.feed_forward.forward(h2 if self.feed_forward.takes_scaled_rows else as_rows(h2), ctx)
+
+
+class HyperConnectionBlock(Block):
+    """A pre-norm layer over a residual that runs in S streams X[:, s] (csrc/streams.hip).  For sublayer q (1: the
+    mixer, 2: the feed-forward, if the layer has one):
+
+        u = sum_s in_q[s] X[s];   y = sublayer(norm_q(u));   X'[t] = sum_s mix_q[s, t] X[s] + out_q[t] y
+
+    with all streams written at once from the old ones.  Tensors: prefix + "hc<q>.in" [S], ".out" [S], ".mix" [S, S]
+    (from, to).  Nothing is left pending: the block's last sum is made inside it.
+    """
+    takes_deferred_product = False
+
+    def __init__(self, prefix: str, streams: int, norm1, mixer, norm2=None, feed_forward=None,
+                 names=("hc1.", "hc2.")):
+        if (norm2 is None) != (feed_forward is None):
+            raise ValueError("the second norm and the feed-forward come together")
+        self.prefix, self.streams, self.names = prefix, int(streams), names
+        self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
+        self.hc = [None, None]
+
+    def _parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    @property
+    def capturable(self):
+        return all(getattr(p, "capturable", False) for p in self._parts())
+
+    def _subs(self):
+        return range(2 if self.feed_forward is not None else 1)
+
+    def tensor_specs(self):
+        from ..weights.source import TensorSpec
+        S, specs = self.streams, {}
+        for p in self._parts():
+            specs.update(p.tensor_specs())
+        for q in self._subs():
+            n = self.prefix + self.names[q]
+            specs.update({n + "in": TensorSpec((S,), "gain"), n + "out": TensorSpec((S,), "gain"),
+                          n + "mix": TensorSpec((S, S), "mixing")})
+        return specs
+
+    def load(self, get):
+        for p in self._parts():
+            p.load(get)
+        for q in self._subs():
+            n = self.prefix + self.names[q]
+            self.hc[q] = tuple(get(n + k).float().contiguous() for k in ("in", "out", "mix"))
+
+    def check(self, dtype):
+        for p in self._parts():
+            p.check(dtype)
+
+    def _read(self, norm, resid, in_w, dtype):
+        if hasattr(norm, "read"):
+            return norm.read(resid, in_w, dtype)
+        import torch
+        from ..kernels import ops
+        u = torch.empty((resid.shape[0], resid.shape[2]), dtype=torch.float32, device=resid.device)
+        ops.streams_read_norm(resid, in_w, u)
+        return norm.add_apply(u, None, dtype)
+
+    @staticmethod
+    def _write(resid, hc, y):
+        from ..kernels import ops
+        from .linear import WeightedDeltas
+        terms = y.terms if isinstance(y, WeightedDeltas) else [(as_delta(y), 1.0, None)]
+        ops.streams_update(resid, hc[2], hc[1], terms)
+
+    def forward(self, resid, pending, ctx, cache, owner=True):
+        if pending is not None:
+            raise ValueError("a block over residual streams takes no pending delta")
+        if resid.dim() != 3 or resid.shape[1] != self.streams:
+            raise ValueError(f"the residual has shape {list(resid.shape)}; this block reads {self.streams} streams")
+        h = self._read(self.norm1, resid, self.hc[0][0], ctx.act_dtype)
+        self._write(resid, self.hc[0], self.mixer.forward(h, ctx, cache, owner))
+        if self.feed_forward is not None:
+            h2 = self._read(self.norm2, resid, self.hc[1][0], ctx.act_dtype)
+            self._write(resid, self.hc[1], self.feed_forward.forward(h2, ctx))
+        return None

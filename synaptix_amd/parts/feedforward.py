@@ -26,7 +26,11 @@ class GatedMlp(FeedForward):
     takes_scaled_rows = True
     capturable = True
 
-    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
+    NAMES = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu", names=None):
+        """names: the tensors of the gate, up and down products behind `prefix` (default: NAMES)."""
+        self.names = tuple(names or self.NAMES)
         try:
             ops.activation_code(activation)       # the kernels apply it by its code; an unknown name is refused here
         except ops.KernelError as e:
@@ -36,20 +40,20 @@ class GatedMlp(FeedForward):
         self.paired = False      # gate and up rows in turns of 16: the activation runs inside the product
 
     def tensor_specs(self):
-        p = self.prefix
+        p, (gate, up, down) = self.prefix, self.names
         return {
-            p + "gate_proj.weight": TensorSpec((self.intermediate, self.hidden)),
-            p + "up_proj.weight": TensorSpec((self.intermediate, self.hidden)),
-            p + "down_proj.weight": TensorSpec((self.hidden, self.intermediate)),
+            p + gate: TensorSpec((self.intermediate, self.hidden)),
+            p + up: TensorSpec((self.intermediate, self.hidden)),
+            p + down: TensorSpec((self.hidden, self.intermediate)),
         }
 
     def load(self, get):
         p = self.prefix
-        gate, up = get(p + "gate_proj.weight"), get(p + "up_proj.weight")
+        gate, up = get(p + self.names[0]), get(p + self.names[1])
         self.paired = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
                        and self.intermediate % ops.PAIR == 0 and self.hidden % 8 == 0)
         self.w_gate_up = Matrix(ops.pair_rows(gate, up) if self.paired else torch.cat([gate, up], 0))
-        self.w_down = Matrix(get(p + "down_proj.weight"))
+        self.w_down = Matrix(get(p + self.names[2]))
 
     def forward(self, h, ctx):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)

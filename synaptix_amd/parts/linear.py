@@ -83,9 +83,28 @@ class DeferredProduct:
         return linear_for_sum(self.x, self.w)
 
 
+class WeightedDeltas:
+    """A sublayer's result that is a sum of one or two scaled terms which have not been added yet:
+    sum_i scale_i * (term_i + bias_i), each term a float tensor [N, hidden] or partial sums [P, N, hidden], each
+    bias float [hidden] or None (two mixers side by side; a last product whose bias is still to come).  A block
+    that says `takes_weighted_deltas` adds them while it writes the residual; everything else asks for `run()`."""
+
+    def __init__(self, terms):
+        self.terms = [(as_delta(t), float(c), b) for t, c, b in terms]
+        first = self.terms[0][0]
+        self.shape = tuple(first.shape[-2:])
+
+    def run(self):
+        first = self.terms[0][0]
+        zero = torch.zeros(self.shape, dtype=torch.float32, device=first.device)
+        one = torch.ones((1,), dtype=torch.float32, device=first.device)
+        ops.streams_update(zero, one.view(1, 1), one, self.terms)
+        return zero
+
+
 def as_delta(d):
     """The delta of the residual rows as a tensor (or None), whatever form it arrives in."""
-    return d.run() if isinstance(d, DeferredProduct) else d
+    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas)) else d
 
 
 def deferred_product(x, w):

@@ -15,7 +15,8 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part, KvNeed
-from .linear import Matrix, linear, linear_for_sum, product_slices, deferred_product, as_rows, ScaledRows
+from .linear import (Matrix, linear, linear_for_sum, product_slices, deferred_product, as_rows, ScaledRows,
+                     WeightedDeltas)
 from .position import Position, NoPosition
 
 
@@ -173,3 +174,157 @@ class GqaAttention(Mixer):
                                           nh, nkv, hd, **terms)
                 o.index_copy_(0, rows, o1)
         return deferred_product(o, self.w_o)
+
+
+def _projection(w):
+    """A projection's weight as the products keep it: in fragment order only where the tiles for many rows read that
+    order too (K a multiple of 128); other widths stay in plain rows."""
+    return Matrix(w, keep_rows=w.shape[1] % 128 != 0)
+
+
+class GatedWindowAttention(Mixer):
+    """Grouped-query attention whose scores, mask and softmax are parameters (csrc/attention_window.hip):
+
+        score(i, j) = scale q_i.k_j [soft cap] + what the position scheme puts on the scores
+        key j is seen by i iff j <= i and (window is None or i - j < window or j < keep_first)
+        p_j = exp(score_j) / (sink + sum exp(score_j)),  sink = 1 with sink_one
+
+    Keys have `dim` values, values `v_dim`.  q, k and v may carry a bias (`bias`), the output product one of its own
+    (`out_bias`); q and k heads may be normed (RMS over the head, one gain for all heads: `qk_norm_eps`); with `gate`
+    the heads' results are multiplied by sigmoid(W_g h) before the output product.  The position scheme may rotate
+    nothing here: it acts on the scores (Position.score_slopes, Position.score_log_bias).  Scores, weights and the
+    norms are 32-bit in both engine types.
+
+    Tensor names: prefix + "q", "k", "v", "o" (+ ".b" for their biases), "q.norm", "k.norm", "g"; `names` renames them.
+    """
+    takes_scaled_rows = False
+    capturable = False      # (its steps are launched one by one)
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": ".b"}
+
+    def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, dim: int, v_dim: int | None = None, *,
+                 position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
+                 window: int | None = None, keep_first: int = 0, sink_one: bool = False, bias: bool = False,
+                 out_bias: bool = False, gate: bool = False, score_softcap: float | None = None, names: dict | None = None):
+        if n_kv_heads <= 0 or n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
+        self.prefix, self.hidden = prefix, hidden
+        self.nh, self.nkv, self.dim, self.vdim = n_heads, n_kv_heads, dim, v_dim or dim
+        self.position = position or NoPosition()
+        self.qk_norm_eps = qk_norm_eps
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(dim)
+        self.window, self.keep_first, self.sink_one = window, int(keep_first or 0), bool(sink_one)
+        self.bias, self.out_bias, self.gate = bool(bias), bool(out_bias), bool(gate)
+        self.score_softcap = float(score_softcap) if score_softcap else 0.0
+        self.names = dict(self.NAMES, **(names or {}))
+        self.w_in = self.w_o = self.b_in = self.b_o = self.q_gain = self.k_gain = None
+        self._terms = None
+
+    def _n(self, key, bias=False):
+        return self.prefix + self.names[key] + (self.names["bias"] if bias else "")
+
+    def _widths(self):
+        return [("q", self.nh * self.dim), ("k", self.nkv * self.dim), ("v", self.nkv * self.vdim)] + \
+               ([("g", self.nh * self.vdim)] if self.gate else [])
+
+    def tensor_specs(self):
+        specs = {self._n(k): TensorSpec((n, self.hidden)) for k, n in self._widths()}
+        specs[self._n("o")] = TensorSpec((self.hidden, self.nh * self.vdim))
+        if self.bias:
+            for k, n in self._widths()[:3]:
+                specs[self._n(k, True)] = TensorSpec((n,), "bias")
+        if self.out_bias:
+            specs[self._n("o", True)] = TensorSpec((self.hidden,), "bias")
+        if self.qk_norm_eps is not None:
+            specs[self._n("q_norm")] = TensorSpec((self.dim,), "gain")
+            specs[self._n("k_norm")] = TensorSpec((self.dim,), "gain")
+        specs.update(self.position.tensor_specs())
+        return specs
+
+    def load(self, get):
+        # one product for q, k, v and the gate: rows of the matrices one after another
+        self.w_in = _projection(torch.cat([get(self._n(k)) for k, _ in self._widths()], 0))
+        self.w_o = _projection(get(self._n("o")))
+        if self.bias:
+            self.b_in = torch.cat([get(self._n(k, True)).float() for k, _ in self._widths()[:3]]).contiguous()
+        if self.out_bias:
+            self.b_o = get(self._n("o", True)).float().contiguous()
+        if self.qk_norm_eps is not None:
+            self.q_gain = get(self._n("q_norm")).float().contiguous()
+            self.k_gain = get(self._n("k_norm")).float().contiguous()
+        self.position.load(get)
+
+    def cache_need(self):
+        return KvNeed(self.nkv, self.dim, self.window, v_dim=self.vdim, keep_first=self.keep_first if self.window else 0)
+
+    def check(self, dtype):
+        if max(self.dim, self.vdim) > ops.WINDOW_ATTENTION_MAX_DIM:
+            raise ValueError(f"{self.prefix}: head sizes {self.dim} and {self.vdim} (at most {ops.WINDOW_ATTENTION_MAX_DIM})")
+        cos, _ = self.position.tables("cpu")
+        if cos is not None:
+            raise ValueError(f"{self.prefix}: this attention takes position schemes that act on the scores, not rotations")
+
+    def _score_terms(self, device):
+        if self._terms is None:
+            sl = self.position.score_slopes(self.nh, device)
+            self._terms = dict(slopes=None if sl is None else sl.to(device=device, dtype=torch.float32).contiguous(),
+                               log_bias=self.position.score_log_bias(self.nh, device), softcap=self.score_softcap)
+        return self._terms
+
+    def forward(self, h, ctx, cache, owner=True):
+        N, act = h.shape[0], h.dtype
+        proj = linear(h, self.w_in, torch.float32)          # [N, q | k | v | gate] float
+        q = torch.empty((N, self.nh * self.dim), dtype=act, device=h.device)
+        table = ctx.page_table(cache.group)
+        ops.window_intake(proj, self.b_in, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
+                          self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, self.nh, self.nkv, self.dim, self.vdim,
+                          write_kv=owner)
+        o = torch.empty((N, self.nh * self.vdim), dtype=act, device=h.device)
+        gate = proj[:, (self.nh + self.nkv) * self.dim + self.nkv * self.vdim:] if self.gate else None
+        ops.window_attention(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, self.nh,
+                             self.nkv, self.dim, self.vdim, window=self.window or 0, keep_first=self.keep_first,
+                             sink_one=self.sink_one, gate=gate, **self._score_terms(h.device))
+        y = linear_for_sum(o, self.w_o)
+        return WeightedDeltas([(y, 1.0, self.b_o)]) if self.b_o is not None else y
+
+
+class ParallelMixers(Mixer):
+    """Several mixers side by side that read the same input; the result is sum_i scale_i * mixer_i(h).  Each keeps
+    what it needs for a sequence: the cache need is the tuple of theirs, and so is the cache view."""
+    takes_scaled_rows = False
+
+    def __init__(self, mixers: list, scales: list):
+        if len(mixers) != len(scales) or not mixers:
+            raise ValueError("one scale for each of the mixers")
+        self.mixers, self.scales = list(mixers), [float(s) for s in scales]
+
+    @property
+    def capturable(self):
+        return all(getattr(m, "capturable", False) for m in self.mixers)
+
+    def tensor_specs(self):
+        specs = {}
+        for m in self.mixers:
+            specs.update(m.tensor_specs())
+        return specs
+
+    def load(self, get):
+        for m in self.mixers:
+            m.load(get)
+
+    def check(self, dtype):
+        for m in self.mixers:
+            m.check(dtype)
+
+    def cache_need(self):
+        return tuple(m.cache_need() for m in self.mixers)
+
+    def forward(self, h, ctx, cache, owner=True):
+        terms = []
+        for m, s, c in zip(self.mixers, self.scales, cache):
+            y = m.forward(h, ctx, c, owner)
+            if isinstance(y, WeightedDeltas):
+                terms += [(t, s * w, b) for t, w, b in y.terms]
+            else:
+                terms.append((y, s, None))
+        return WeightedDeltas(terms)

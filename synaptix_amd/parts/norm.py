@@ -58,3 +58,46 @@ class RmsNorm(Part):
         out = torch.empty_like(x)
         ops.rmsnorm_rows(x, self.gain, self.eps, out, self.gain_offset)
         return out
+
+
+class DynamicTanh(Part):
+    """y = tanh(alpha * x) * gain + shift with a scalar alpha: a norm that takes no mean and no variance.
+
+    Tensors: `name` (gain [dim]), `name + alpha_suffix` (one number), `name + shift_suffix` ([dim]).  Arithmetic in
+    32-bit.  The residual it reads may run in several streams [N, S, dim]: `add_apply` then norms their sum, or with
+    `read` a weighted sum of them (what a block with hyper-connections hands its sublayers).
+    """
+    capturable = True
+    takes_deferred_product = False
+
+    def __init__(self, name: str, dim: int, alpha_suffix: str = ".alpha", shift_suffix: str = ".b"):
+        self.name, self.dim = name, dim
+        self.alpha_name, self.shift_name = name + alpha_suffix, name + shift_suffix
+        self.gain = self.alpha = self.shift = None
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.dim,), "gain"), self.alpha_name: TensorSpec((), "gain"),
+                self.shift_name: TensorSpec((self.dim,), "bias")}
+
+    def load(self, get):
+        # a few hundred numbers: kept in 32-bit whatever the engine's type
+        self.gain = get(self.name).float().contiguous()
+        self.alpha = get(self.alpha_name).float().reshape(1).contiguous()
+        self.shift = get(self.shift_name).float().contiguous()
+
+    def read(self, resid, in_weights, out_dtype, rows=None, delta=None):
+        """The norm of sum_s in_weights[s] * resid[:, s] (in_weights None: of the sum of the streams)."""
+        n = resid.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((n, self.dim), dtype=out_dtype, device=resid.device)
+        ops.streams_read_norm(resid, in_weights, out, dyt=(self.alpha, self.gain, self.shift), rows=rows, delta=delta)
+        return out
+
+    def add_apply(self, resid, delta, out_dtype, rows=None):
+        """As RmsNorm.add_apply; a residual in several streams comes without a delta and is summed over its streams."""
+        return self.read(resid, None, out_dtype, rows=rows, delta=delta)
+
+    def apply(self, x):
+        out = torch.empty_like(x)
+        x32 = x if x.dtype == torch.float32 else x.float()
+        ops.streams_read_norm(x32.reshape(-1, self.dim), None, out.view(-1, self.dim), dyt=(self.alpha, self.gain, self.shift))
+        return out

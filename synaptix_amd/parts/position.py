@@ -24,6 +24,11 @@ class Position(Part):
         crates/synaptix-ops/src/pos/alibi.rs:47-66); None (the default): nothing is added."""
         return None
 
+    def score_log_bias(self, n_heads: int, device):
+        """A scheme whose term on the scores grows with the logarithm of the distance: (r1, r2), float [n_heads] each
+        on `device`, for - r1[head] * ln(1 + r2[head] * (p - j)); None (the default): nothing is added."""
+        return None
+
     capacity = None  # positions at and beyond it cannot be encoded; None: no limit
 
 
@@ -57,3 +62,28 @@ class RotaryHalfSplit(Position):
             cos, sin = self.host_tables()
             self._tables[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))
         return self._tables[key]
+
+
+class LogDistanceBias(Position):
+    """No rotation; the score of query position i and key position j <= i gets  - r1[h] * ln(1 + r2[h] * (i - j)),
+    with one pair of numbers a head, read from the tensors `prefix + r1_name` and `prefix + r2_name` ([n_heads])."""
+    capturable = True
+
+    def __init__(self, prefix: str, n_heads: int, r1_name: str = "r1", r2_name: str = "r2"):
+        self.n_heads = n_heads
+        self.r1_name, self.r2_name = prefix + r1_name, prefix + r2_name
+        self.r1 = self.r2 = None
+
+    def tensor_specs(self):
+        from ..weights.source import TensorSpec
+        return {self.r1_name: TensorSpec((self.n_heads,), "positive"), self.r2_name: TensorSpec((self.n_heads,), "positive")}
+
+    def load(self, get):
+        self.r1 = get(self.r1_name).float().contiguous()
+        self.r2 = get(self.r2_name).float().contiguous()
+
+    def score_log_bias(self, n_heads: int, device):
+        """(r1, r2) float [n_heads] on the device."""
+        if n_heads != self.n_heads:
+            raise ValueError(f"a distance bias for {self.n_heads} heads was asked for {n_heads}")
+        return self.r1, self.r2

@@ -42,7 +42,7 @@ class Pipeline:
             raise ValueError(f"device {device!r}: this engine runs on the GPU only")
         from .config import load_config
         _, cfg = load_config(path)
-        longest = max_seq or cfg.max_position_embeddings
+        longest = max_seq or getattr(cfg, "max_position_embeddings", None) or 4096
         if max_tokens is None:
             max_tokens = min(8 * longest, 65536)
             max_tokens = max(max_tokens, longest)
@@ -64,7 +64,7 @@ class Pipeline:
         with open(config_json) as f:
             d = json.load(f)
         cfg = resolve_architecture(d).config_cls.from_dict(d)
-        longest = max_seq or cfg.max_position_embeddings
+        longest = max_seq or getattr(cfg, "max_position_embeddings", None) or 4096
         if max_tokens is None:
             max_tokens = max(min(8 * longest, 65536), longest)
         eng = Engine.from_config(cfg, seed=seed, dtype=_DTYPE_NAMES[dtype], max_tokens=max_tokens, max_slots=max_batch,

@@ -16,7 +16,8 @@ from .safetensors_io import SafetensorsFile, resolve_shards, _NAMES
 @dataclass(frozen=True)
 class TensorSpec:
     """What a part expects under a name.  `kind` only matters to the random generator:
-    "matrix" and "table" draw N(0, std), "gain" draws 1 + N(0, gain_std)."""
+    "matrix" and "table" draw N(0, std), "gain" draws 1 + N(0, gain_std), "bias" N(0, gain_std), "positive"
+    |N(0, 1)| / 2 + 0.05, "mixing" (a square matrix) the identity + N(0, gain_std)."""
     shape: tuple
     kind: str = "matrix"
 
@@ -113,6 +114,13 @@ class RandomSource(WeightSource):
         shape = tuple(spec.shape)
         if spec.kind == "gain":
             t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std + 1.0
+        elif spec.kind == "bias":
+            t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std
+        elif spec.kind == "positive":
+            t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32).abs() * 0.5 + 0.05
+        elif spec.kind == "mixing":
+            t = (torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std
+                 + torch.eye(shape[0], device=self.device))
         elif self.device.type == "cpu" or self.store_dtype == torch.float32:
             t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.std
         else:
