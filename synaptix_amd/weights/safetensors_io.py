@@ -123,5 +123,5 @@ def save_file(tensors: dict, path: str, metadata: dict | None = None) -> None:
         f.write(raw)
         for t in blobs:
             if t.numel():
-                f.write(t.view(torch.uint8).numpy().tobytes() if t.dtype != torch.bool
+                f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.dtype != torch.bool      # (a scalar has no axis to view)
                         else t.to(torch.uint8).numpy().tobytes())

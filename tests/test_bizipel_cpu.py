@@ -1,0 +1,141 @@
+"""Bizipel without a GPU: its configuration and registry entry, the tensors it declares, what its layers ask of the
+cache (keys and values beside a running state; first keys that a window keeps), and the plain model's own mechanisms."""
+import copy
+
+import pytest
+import torch
+
+import plain_bizipel as P
+from bizipel_cases import CONFIGS, layer, config
+from synaptix_amd.cache import SequenceCache, pages_for
+from synaptix_amd.config import BizipelConfig, ConfigError, resolve_architecture
+from synaptix_amd.parts import KvNeed, StateNeed
+
+
+def test_configuration_round_trip_and_registry():
+    for name, d in CONFIGS.items():
+        arch = resolve_architecture(d)
+        assert arch.name == "Bizipel"
+        cfg = arch.config_cls.from_dict(copy.deepcopy(d))
+        assert BizipelConfig.from_dict(cfg.to_dict()) == cfg
+        assert len(cfg.layers) == len(d["layers"]) and cfg.vocab_size == d["vocab"]
+    cfg = BizipelConfig.from_dict(CONFIGS["P"])
+    assert cfg.layers[0].left.window == 20 and cfg.layers[0].left.keep_first == 3 and cfg.layers[1].ff is None
+    assert cfg.streams == 2 and BizipelConfig.from_dict(CONFIGS["Q"]).streams == 1
+    assert BizipelConfig.from_dict(config(10, 8, None, [layer(1, 1, 4, 4, 8, 0, 1, 4, 4, 8)])).streams is None
+
+
+@pytest.mark.parametrize("change,match", [
+    (lambda d: d["layers"][0].__setitem__("type", "serial"), "layer type"),
+    (lambda d: d["layers"][0]["mixer"]["left"].__setitem__("kv_heads", 3), "divisible"),
+    (lambda d: d["layers"][0]["mlp"].__setitem__("kind", "routed"), "dense"),
+    (lambda d: d["layers"][0]["mixer"]["right"].__setitem__("gate_cap", 0), "gate_cap"),
+    (lambda d: d["layers"][0]["mixer"]["left"].pop("mask"), "mask"),
+    (lambda d: d.__setitem__("width", 0), "width"),
+    (lambda d: d.__setitem__("layers", []), "layers"),
+    (lambda d: d["norm"].__setitem__("eps", "tiny"), "eps"),
+])
+def test_configuration_names_what_is_wrong(change, match):
+    d = copy.deepcopy(CONFIGS["P"])
+    change(d)
+    with pytest.raises(ConfigError, match=match):
+        BizipelConfig.from_dict(d)
+
+
+def test_the_model_declares_its_tensors_and_cache_needs():
+    arch = resolve_architecture(CONFIGS["P"])
+    model = arch.build(arch.config_cls.from_dict(CONFIGS["P"]))
+    specs = model.tensor_specs()
+    assert specs["embed"].shape == (300, 64) and specs["final.norm.alpha"].shape == ()
+    assert specs["l0.mix.left.q"].shape == (4 * 16, 64) and specs["l0.mix.left.v.b"].shape == (2 * 24,)
+    assert specs["l0.mix.left.g"].shape == (4 * 24, 64) and specs["l0.mix.left.o"].shape == (64, 4 * 24)
+    assert specs["l0.mix.right.i"].shape == (2, 64) and specs["l0.mix.right.norm"].shape == (2 * 16,)
+    assert specs["l0.hc2.mix"].shape == (2, 2) and specs["l1.hc1.in"].shape == (2,)
+    assert not any(n.startswith(("l1.mlp", "l1.norm2", "l1.hc2")) for n in specs)        # a layer without a feed-forward
+    needs = model.cache_needs()
+    assert needs[0] == (KvNeed(2, 16, 20, v_dim=24, keep_first=3), StateNeed((2, 8 * 16 + 8 + 1)))
+    assert needs[1] == (KvNeed(1, 32, 70, v_dim=16, keep_first=0), StateNeed((1, 24 * 40 + 24 + 1)))
+    assert model.streams == 2 and not model.capturable()
+
+
+def test_a_cache_layer_may_hold_keys_and_a_state():
+    needs = [(KvNeed(2, 16, 20, v_dim=24, keep_first=3), StateNeed((2, 9))), KvNeed(2, 16), (StateNeed((4,)),)]
+    c = SequenceCache(needs, 640, 4, torch.float32, "cpu")
+    kv, st = c.layer_view(0)
+    assert kv.k_pages.shape == (11, 2, 64, 16) and kv.v_pages.shape == (11, 2, 24, 64) and st.state.shape == (5, 2, 9)
+    assert c.layer_view(1).v_pages.shape == (11, 2, 16, 64) and c.layer_view(2)[0].state.shape == (5, 4)
+    a = c.acquire()
+    st.state[a] += 1.0
+    snap = c.snapshot(a)
+    st.state[a] += 1.0
+    c.restore(snap)
+    assert float(st.state[a].min()) == 1.0
+    c.release(a)
+    assert c.acquire() == a and float(st.state[a].abs().max()) == 0.0       # zero again when the slot is taken again
+    c.check()
+
+
+def test_a_window_never_gives_back_the_pages_of_its_kept_first_keys():
+    window, keep = 70, 65                   # the kept keys reach into the second page
+    c = SequenceCache([KvNeed(1, 8, window, keep_first=keep), KvNeed(1, 8, window)], 64 * 12, 2, torch.float32, "cpu")
+    s = c.acquire()
+    c.reserve(s, 500)
+    c.commit(s, 500)
+    first_needed = (500 - window + 1) // 64
+    free_kept, free_plain = c.groups[0].pool.free_pages, c.groups[1].pool.free_pages
+    assert free_plain - free_kept == pages_for(keep)                 # two pages more are held for good
+    assert free_plain == 12 - (pages_for(500) - first_needed)
+    for _ in range(300):
+        c.reserve(s, 1)
+        c.commit(s, 1)
+    assert c.groups[1].pool.free_pages - c.groups[0].pool.free_pages == pages_for(keep)
+    c.truncate(s, 790)
+    c.release(s)
+    assert c.groups[0].pool.free_pages == 12 == c.groups[1].pool.free_pages
+    c.check()
+
+
+def test_planning_counts_the_kept_pages():
+    c = SequenceCache([KvNeed(1, 8, 100, keep_first=130)], 64 * 64, 4, torch.float32, "cpu", max_step_tokens=64)
+    assert c.pages_for_sequence(4000, 64) == [pages_for(100 + 64) + 1 + pages_for(130)]
+    assert c.groups[0].n_pages == 4 * (pages_for(164) + 1 + 3)
+
+
+# ----------------------------------------------------------------------------- the plain model's own mechanisms
+
+def test_plain_mask_window_and_kept_keys():
+    seen = P.visible(12, 4, 2)
+    assert seen[11].tolist() == [True, True] + [False] * 6 + [True] * 4
+    assert seen[3].tolist() == [True] * 4 + [False] * 8 and seen[5].tolist() == [True, True, True, True, True, True] + [False] * 6
+    assert P.visible(5, None, 0).tolist() == torch.tril(torch.ones(5, 5)).bool().tolist()
+
+
+def test_plain_attention_sink_takes_weight_and_distance_lowers_scores():
+    q = torch.zeros(3, 1, 2, dtype=P.F64)
+    k = torch.zeros(3, 1, 2, dtype=P.F64)
+    v = torch.ones(3, 1, 1, dtype=P.F64)
+    out = P.window_attention(q, k, v, 1.0, None, 0)            # all scores 0: i + 1 keys and the sink share the weight
+    assert torch.allclose(out[:, 0, 0], torch.tensor([1 / 2, 2 / 3, 3 / 4], dtype=P.F64))
+    out = P.window_attention(q, k, v, 1.0, None, 0, sink_one=False)
+    assert torch.allclose(out[:, 0, 0], torch.ones(3, dtype=P.F64))
+    r1, r2 = torch.tensor([2.0], dtype=P.F64), torch.tensor([1.0], dtype=P.F64)
+    out = P.window_attention(q, k, v, 1.0, None, 0, r1, r2)    # exp(-2 ln(1 + d)) = (1 + d)^-2
+    assert torch.allclose(out[2, 0, 0], torch.tensor((1 + 1 / 4 + 1 / 9) / (2 + 1 / 4 + 1 / 9), dtype=P.F64))
+
+
+def test_plain_matrix_memory_in_two_pieces_equals_one_and_stays_finite():
+    g = torch.Generator().manual_seed(0)
+    T, H, D, E = 40, 2, 5, 7
+    q, k = torch.randn(T, H, D, generator=g, dtype=P.F64), torch.randn(T, H, D, generator=g, dtype=P.F64)
+    v = torch.randn(T, H, E, generator=g, dtype=P.F64)
+    ip, fp = 30 * torch.randn(T, H, generator=g, dtype=P.F64), 30 * torch.randn(T, H, generator=g, dtype=P.F64)
+    whole, _ = P.matrix_memory(q, k, v, ip, fp, 12.0)
+    a, st = P.matrix_memory(q[:13], k[:13], v[:13], ip[:13], fp[:13], 12.0)
+    b, _ = P.matrix_memory(q[13:], k[13:], v[13:], ip[13:], fp[13:], 12.0, st)
+    assert torch.allclose(torch.cat([a, b]), whole, rtol=1e-12, atol=1e-12) and torch.isfinite(whole).all()
+    # one step by hand: m_1 = max(f + 0, i); C = e^(i - m) k v^T; o = C^T q / (max(|n.q|, e^-m) + 1e-6)
+    o, (C, n, m) = P.matrix_memory(q[:1], k[:1], v[:1], ip[:1], fp[:1], 12.0)
+    li = 12.0 * torch.tanh(ip[0] / 12.0)
+    lf = torch.nn.functional.logsigmoid(12.0 * torch.tanh(fp[0] / 12.0))
+    assert torch.allclose(m, torch.maximum(lf, li))
+    assert torch.allclose(n, torch.exp(li - m)[:, None] * k[0])
