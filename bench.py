@@ -2,6 +2,7 @@
 """Throughput of the engine at a Qwen3 shape with random bf16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|4b|32b] [--batch 8] [--layers L]
+    python bench.py --design bizipel [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
 
 --shape 8b (the default) and 32b: a step is one decode step of `batch` sequences, each after a
 2,048-token prompt of uniform ids, run through the same captured graph and host loop that
@@ -20,6 +21,10 @@ The default run (8b, without --no-points) measures the other workloads as well a
 own clock over its last `steps` decode steps, to stand beside `value`), the 4b workload
 (decode_4b_unequal16, its fraction of the HBM roofline and its prompts' rate) and the 32b shape at
 8 sequences (decode_32b_b8), each with the sizes it ran at as a text.
+
+--design bizipel: not the contract's run.  Prefill and decode throughput of the Bizipel design at a few layer sizes
+beside the Qwen3 decoder at the same sizes (width, heads, head size, feed-forward, vocabulary, layers; random bf16
+weights), each with the time of every kernel entry point of one prompt step and one decode step; one JSON line.
 
 Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
 crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
@@ -161,6 +166,107 @@ def through_generate(eng, cfg, batch, prompt_len, warmup, steps, weight_bytes, u
     step_bytes = weight_bytes + batch * mean_ctx * eng.cache.bytes_per_token()
     return batch / step_s, step_s, step_bytes
 
+# ----------------------------------------------------------------------------- two designs side by side
+DESIGN_SIZES = {     # layers, width, heads, kv heads, head size, feed-forward, vocabulary
+    "small": (4, 1024, 8, 8, 128, 4096, 32768),
+    "mid": (4, 2048, 16, 8, 128, 8192, 32768),
+    "large": (4, 4096, 32, 8, 128, 12288, 32768),
+}
+
+
+def design_configs(size, window, context):
+    """(Qwen3 configuration, Bizipel configuration) of one size: the same width, attention heads, feed-forward,
+    vocabulary (tied) and number of layers; the Bizipel layers add a matrix memory of heads / 4 heads (keys of 64,
+    values of 128), two residual streams and a window that keeps 4 first keys."""
+    from synaptix_amd import Qwen3Config
+    from synaptix_amd.config import BizipelConfig
+    L, W, nh, nkv, hd, ff, V = DESIGN_SIZES[size]
+    qwen = Qwen3Config.from_dict(dict(_COMMON, num_hidden_layers=L, hidden_size=W, num_attention_heads=nh,
+                                      num_key_value_heads=nkv, head_dim=hd, intermediate_size=ff, vocab_size=V,
+                                      tie_word_embeddings=True, max_position_embeddings=context))
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                "mask": {"size": window, "keep_first": 4}},
+                       "right": {"heads": max(1, nh // 4), "dim": 64, "vdim": 128, "gate_cap": 15.0},
+                       "left_scale": 1.0, "right_scale": 1.0},
+             "mlp": {"kind": "dense", "ff": ff}}
+    biz = BizipelConfig.from_dict({"architecture": "Bizipel", "vocab": V, "width": W, "streams": 2, "norm": {"eps": 1e-6},
+                                   "layers": [layer] * L})
+    return qwen, biz
+
+
+def designs_side_by_side(args) -> int:
+    import torch
+    from synaptix_amd import Engine
+    from synaptix_amd.kernels import ops
+    sizes = [s for s in args.sizes.split(",") if s]
+    for s in sizes:
+        if s not in DESIGN_SIZES:
+            print(f"bench.py: --sizes names {s!r}; known: {', '.join(DESIGN_SIZES)}")
+            return 2
+    P, B = args.prompt, args.batch
+    steps, warmup = (args.steps or 32), min(args.warmup, 8)
+    context = P + steps + warmup + 72
+    points = {}
+    for size in sizes:
+        for design, cfg in zip(("qwen3", "bizipel"), design_configs(size, args.window, context)):
+            torch.manual_seed(0)
+            eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=(B + 1) * ((context + 63) // 64 * 64),
+                                     max_seq=context if design == "qwen3" else None)
+            weight_bytes = sum(2 * int(torch.Size(sp.shape).numel()) for sp in eng.model.tensor_specs().values())
+            g = torch.Generator().manual_seed(0)
+            prompt = torch.randint(0, cfg.vocab_size, (P,), generator=g).tolist()
+            times = []
+            for i in range(4):                       # the first one warms up (and builds what is built at first use)
+                s = eng.acquire()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.step([(s, prompt)], want="last")
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                if i == 3:
+                    with ops.op_timing() as table:   # the same step once more, every entry point timed alone
+                        eng.restore(snap)
+                        eng.step([(s, prompt)], want="last")
+                    prefill_ops = {k: round(v[0], 3) for k, v in sorted(table.items(), key=lambda kv: -kv[1][0])[:8]}
+                eng.release(s)
+                if i == 2:
+                    s = eng.acquire()
+                    snap = eng.snapshot(s)
+                    eng.release(s)
+            pre_s = min(times[1:])
+            rate, step_s, step_bytes = through_generate(eng, cfg, B, P, warmup, steps, weight_bytes,
+                                                        use_graph=not args.no_graph)
+            slots = [eng.acquire() for _ in range(B)]
+            eng.step([(s, prompt) for s in slots], want="last")
+            with ops.op_timing() as table:
+                eng.step([(s, [1]) for s in slots], want="last")
+            decode_ops = {k: round(v[0], 3) for k, v in sorted(table.items(), key=lambda kv: -kv[1][0])[:8]}
+            key = f"{size}_{design}"
+            points[key + "_prefill_tok_s"] = round(P / pre_s, 1)
+            points[key + "_prefill_ms"] = round(pre_s * 1e3, 3)
+            points[key + f"_decode_b{B}_tok_s"] = round(rate, 1)
+            points[key + f"_decode_b{B}_ms_per_step"] = round(step_s * 1e3, 4)
+            points[key + f"_decode_b{B}_hbm_frac"] = round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
+            points[key + "_prefill_ops_ms"] = json.dumps(prefill_ops)
+            points[key + "_decode_ops_ms"] = json.dumps(decode_ops)
+            del eng
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+    first = sizes[0]
+    line = {"metric": f"decode tok/s at batch {B} of the Bizipel design at the {first} size (the Qwen3 decoder at equal sizes "
+                      f"and prefill at {P} tokens in points), bf16", "value": points[f"{first}_bizipel_decode_b{B}_tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": points[f"{first}_bizipel_decode_b{B}_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
+            "config": {"model": "Bizipel beside Qwen3 at equal layer sizes", "sizes": {s: list(DESIGN_SIZES[s]) for s in sizes},
+                       "global_batch": B, "seq_len": P, "window": args.window, "parallelism": "single GPU",
+                       "graph": not args.no_graph},
+            "points": points}
+    print(json.dumps(line))
+    return 0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -177,7 +283,16 @@ def main() -> int:
                     help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
+    ap.add_argument("--design", default=None, choices=["bizipel"],
+                    help="not the contract's run: this design beside the Qwen3 decoder at equal layer sizes")
+    ap.add_argument("--sizes", default="small,mid,large", help="with --design: which of small, mid, large")
+    ap.add_argument("--window", type=int, default=1024, help="with --design: the keys a query of the new design sees")
     args = ap.parse_args()
+    if args.design is not None:
+        if args.gpus != 1:
+            print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+            return 2
+        return designs_side_by_side(args)
     shape = SHAPES[args.shape]
     if args.steps is None:
         args.steps = 127 if args.shape == "4b" else 128

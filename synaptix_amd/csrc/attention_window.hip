@@ -110,34 +110,41 @@ __device__ __forceinline__ float window_score(float dot, float scale, const Wind
   return s;
 }
 
-template <typename T>
-__global__ void __launch_bounds__(SYN_WAVE)
+// WAVES waves a (token, head): wave w takes every WAVES-th of the visible blocks of 64 keys, and the waves' partial
+// results (maximum, sum, weighted values) are merged through LDS at the end.  One wave is enough where a step has many
+// tokens; single tokens over a long window get eight.
+template <typename T, int WAVES>
+__global__ void __launch_bounds__(WAVES * SYN_WAVE)
 window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                         const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                         const int* __restrict__ tok_pos, const float* __restrict__ gate, int gate_stride,
                         const float* __restrict__ gate_bias, T* __restrict__ out, float scale, int nh, int nkv, int dim,
                         int vdim, WindowTerms terms) {
   __shared__ float qs[AW_MAX_DIM];
-  __shared__ float ps[SYN_PAGE];
-  const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  __shared__ float ps[WAVES][SYN_PAGE];
+  __shared__ float part_o[WAVES][AW_MAX_DIM];
+  __shared__ float part_ml[WAVES][2];
+  const int tok = blockIdx.x, head = blockIdx.y;
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int seq = tok_seq[tok], pos = tok_pos[tok];
   const int kvh = head / (nh / nkv);
   const T* qr = q + ((size_t)tok * nh + head) * dim;
-  for (int d = lane; d < dim; d += SYN_WAVE) qs[d] = to_f32<T>(qr[d]);
+  for (int d = threadIdx.x; d < dim; d += WAVES * SYN_WAVE) qs[d] = to_f32<T>(qr[d]);
   __syncthreads();
 
   const int lo = terms.window > 0 ? max(0, pos - terms.window + 1) : 0;
   const int kept = min(terms.keep_first, lo);        // keys below `kept` are seen although the window has passed them
-  const int last_kept_block = kept > 0 ? (kept - 1) / SYN_PAGE : -1;
-  const int first_window_block = max(lo / SYN_PAGE, last_kept_block + 1);
-  const int last_block = pos / SYN_PAGE;
+  const int n_kept_blocks = kept > 0 ? (kept - 1) / SYN_PAGE + 1 : 0;
+  const int first_window_block = max(lo / SYN_PAGE, n_kept_blocks);
+  const int n_blocks = n_kept_blocks + (pos / SYN_PAGE - first_window_block + 1);
   const float slope = terms.slopes ? terms.slopes[head] : 0.f;
   const float r1 = terms.r1 ? terms.r1[head] : 0.f, r2 = terms.r1 ? terms.r2[head] : 0.f;
-  // the sink is a key of score 0 without a value: the running maximum and sum start from it
-  float m = terms.sink_one ? 0.f : -INFINITY, l = terms.sink_one ? 1.f : 0.f;
+  // the sink is a key of score 0 without a value: the first wave's running maximum and sum start from it
+  const bool sink_here = terms.sink_one && wave == 0;
+  float m = sink_here ? 0.f : -INFINITY, l = sink_here ? 1.f : 0.f;
   float o[AW_MAX_DIM / SYN_WAVE] = {0.f, 0.f, 0.f, 0.f};
-  for (int kb = last_kept_block >= 0 ? 0 : first_window_block; kb <= last_block; ++kb) {
-    if (kb == last_kept_block + 1 && kb < first_window_block) kb = first_window_block;
+  for (int idx = wave; idx < n_blocks; idx += WAVES) {
+    const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
     const int page = page_table[(size_t)seq * table_stride + kb];
     const size_t kbase = ((size_t)page * nkv + kvh) * SYN_PAGE * dim;
     const size_t vbase = ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
@@ -155,8 +162,14 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     const float p = valid ? expf(s - m_new) : 0.f;
     l = l * alpha + wave_sum(p);
     m = m_new;
-    ps[lane] = p;
-    __syncthreads();
+    // the wave's own lanes exchange their weights through LDS: a barrier of the wave, not of the workgroup (the
+    // waves walk different numbers of blocks)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    ps[wave][lane] = p;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
     for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i) {
       const int d = lane + i * SYN_WAVE;
@@ -164,13 +177,33 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
         const T* vr = v_pages + vbase + (size_t)d * SYN_PAGE;
         float acc = o[i] * alpha;
         for (int j = 0; j < SYN_PAGE; ++j) {
-          const float pj = ps[j];
+          const float pj = ps[wave][j];
           if (pj != 0.f) acc = fmaf(pj, to_f32<T>(vr[j]), acc);   // slots past the sequence's end may hold anything
         }
         o[i] = acc;
       }
     }
+  }
+  if (WAVES > 1) {
+    // merge in the waves' order: the largest maximum, every wave's sum and values scaled to it
+    if (lane == 0) part_ml[wave][0] = m, part_ml[wave][1] = l;
+#pragma unroll
+    for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i)
+      if (lane + i * SYN_WAVE < vdim) part_o[wave][lane + i * SYN_WAVE] = o[i];
     __syncthreads();
+    if (wave != 0) return;
+    float mm = -INFINITY;
+    for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, part_ml[w][0]);
+    l = 0.f;
+#pragma unroll
+    for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i) o[i] = 0.f;
+    for (int w = 0; w < WAVES; ++w) {
+      const float f = part_ml[w][0] == -INFINITY ? 0.f : expf(part_ml[w][0] - mm);
+      l += f * part_ml[w][1];
+#pragma unroll
+      for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i)
+        if (lane + i * SYN_WAVE < vdim) o[i] += f * part_o[w][lane + i * SYN_WAVE];
+    }
   }
   T* orow = out + ((size_t)tok * nh + head) * vdim;
   const float* g = gate ? gate + (size_t)tok * gate_stride + (size_t)head * vdim : nullptr;
@@ -205,14 +238,225 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
   SYN_CHECK(gate == nullptr || gate_stride >= nh * vdim, "window_attention: gate rows of %d values", gate_stride);
   const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one};
   const dim3 grid(n_tokens, nh);
-  if (is_f32)
-    window_attention_kernel<float><<<grid, SYN_WAVE, 0, stream>>>(
-        (const float*)q, (const float*)k_pages, (const float*)v_pages, page_table, table_stride, tok_seq, tok_pos, gate,
-        gate_stride, gate_bias, (float*)out, scale, nh, nkv, dim, vdim, terms);
-  else
-    window_attention_kernel<bf16><<<grid, SYN_WAVE, 0, stream>>>(
-        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, tok_seq, tok_pos, gate,
-        gate_stride, gate_bias, (bf16*)out, scale, nh, nkv, dim, vdim, terms);
+  // few (token, head) pairs (single tokens of a few sequences): eight waves share each pair's keys
+  const bool many_waves = (long)n_tokens * nh < 8L * syn_compute_units();
+#define SYN_AW(T, W)                                                                                                  \
+  window_attention_kernel<T, W><<<grid, W * SYN_WAVE, 0, stream>>>((const T*)q, (const T*)k_pages, (const T*)v_pages,   \
+                                                                   page_table, table_stride, tok_seq, tok_pos, gate,   \
+                                                                   gate_stride, gate_bias, (T*)out, scale, nh, nkv, dim, \
+                                                                   vdim, terms)
+  if (is_f32) {
+    if (many_waves) SYN_AW(float, 8); else SYN_AW(float, 1);
+  } else {
+    if (many_waves) SYN_AW(bf16, 8); else SYN_AW(bf16, 1);
+  }
+#undef SYN_AW
   SYN_LAUNCH_CHECK("window_attention");
+  return 0;
+}
+
+// ---------------------------------------------------------------- prompts in bf16 on the matrix cores
+// One wave for 16 queries of one (sequence, head), four such waves a workgroup, no LDS and no barrier: a wave walks
+// the pages its queries see, 64 keys at a time.  S^T = K Q^T (MFMA 16x16: a lane then holds four keys of ONE query, so
+// the softmax's statistics are a lane's own plus two exchanges across the lane groups), and the accumulator's layout
+// is the B operand of O^T += V^T P^T, whose A operand are 8-byte pieces of the V page's rows.  The weights meet V as
+// two bf16 numbers each (the weight rounded, and what the rounding left), so that they count with 16 bits of mantissa
+// although the product runs in bf16.  Head sizes in steps of 16 up to 128 (keys in steps of 32 take k-steps of 32).
+#define AWP_TILES 8
+typedef __attribute__((ext_vector_type(4))) __bf16 awp_bf16x4;
+
+__device__ __forceinline__ f32x4 awp_mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 awp_mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ bf16x8 awp_join(bf16x4 lo, bf16x4 hi) {
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = lo[e], r[4 + e] = hi[e];
+  return r;
+}
+
+template <bool X32>
+__global__ void __launch_bounds__(256)
+window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+                           const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
+                           const int* __restrict__ seq_past, int n_seqs, const float* __restrict__ gate, int gate_stride,
+                           const float* __restrict__ gate_bias, bf16* __restrict__ out, float scale, int nh, int nkv,
+                           int dim, int vdim, WindowTerms terms) {
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, g = lane / 16;
+  int bt = blockIdx.x, seq = -1, n_new = 0, start = 0;
+  for (int b = 0; b < n_seqs; ++b) {
+    const int s0 = seq_start[b], n = seq_start[b + 1] - s0, tiles = (n + 63) / 64;
+    if (bt < tiles) {
+      seq = b, n_new = n, start = s0;
+      break;
+    }
+    bt -= tiles;
+  }
+  if (seq < 0) return;
+  const int n0 = bt * 64 + wave * 16;
+  if (n0 >= n_new) return;
+  const int head = blockIdx.y, kvh = head / (nh / nkv);
+  const int past = seq_past[seq];
+  const bool q_ok = n0 + i < n_new;
+  const int my_n = min(n0 + i, n_new - 1);       // (rows beyond the sequence's tokens repeat its last one and are not stored)
+  const int qpos = past + my_n;
+  const int vt = vdim / 16;
+  const bf16* qrow = q + ((size_t)(start + my_n) * nh + head) * dim;
+  bf16x8 qf8[AWP_TILES / 2];
+  bf16x4 qf4[AWP_TILES];
+  if constexpr (X32) {
+#pragma unroll
+    for (int s = 0; s < AWP_TILES / 2; ++s)
+      if (s < dim / 32) qf8[s] = *(const bf16x8*)(qrow + 32 * s + 8 * g);
+  } else {
+#pragma unroll
+    for (int s = 0; s < AWP_TILES; ++s)
+      if (s < dim / 16) qf4[s] = *(const bf16x4*)(qrow + 16 * s + 4 * g);
+  }
+  const int W = terms.window;
+  const int lo_q = W > 0 ? max(0, qpos - W + 1) : 0;                          // this lane's query
+  const int lo_first = W > 0 ? max(0, past + n0 - W + 1) : 0;                 // the tile's first query
+  const int kmax = past + min(n0 + 15, n_new - 1);
+  const int kept = min(terms.keep_first, lo_first);
+  const int n_kept_blocks = kept > 0 ? (kept - 1) / SYN_PAGE + 1 : 0;
+  const int first_window_block = max(lo_first / SYN_PAGE, n_kept_blocks);
+  const int n_blocks = n_kept_blocks + (kmax / SYN_PAGE - first_window_block + 1);
+  const float slope = terms.slopes ? terms.slopes[head] : 0.f;
+  const float r1 = terms.r1 ? terms.r1[head] : 0.f, r2 = terms.r1 ? terms.r2[head] : 0.f;
+  float m = terms.sink_one ? 0.f : -INFINITY, l = terms.sink_one ? 1.f : 0.f;
+  f32x4 O[AWP_TILES];
+#pragma unroll
+  for (int j = 0; j < AWP_TILES; ++j) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int idx = 0; idx < n_blocks; ++idx) {
+    const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
+    const int page = page_table[(size_t)seq * table_stride + kb];
+    const bf16* kpage = k_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * dim;
+    const bf16* vpage = v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
+    f32x4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* krow = kpage + (size_t)(16 * t + i) * dim;
+      if constexpr (X32) {
+#pragma unroll
+        for (int c = 0; c < AWP_TILES / 2; ++c)
+          if (c < dim / 32) s[t] = awp_mfma32(*(const bf16x8*)(krow + 32 * c + 8 * g), qf8[c], s[t]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < AWP_TILES; ++c)
+          if (c < dim / 16) s[t] = awp_mfma16(*(const bf16x4*)(krow + 16 * c + 4 * g), qf4[c], s[t]);
+      }
+    }
+    // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i)
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = kb * SYN_PAGE + 16 * t + 4 * g + e;
+        const bool valid = key <= qpos && (key >= lo_q || key < terms.keep_first);
+        float v = s[t][e] * scale;
+        if (terms.softcap > 0.f) v = terms.softcap * tanhf(v / terms.softcap);
+        const float dist = (float)(qpos - key);
+        v -= slope * dist;
+        if (terms.r1) v -= r1 * __logf(1.f + r2 * dist);
+        v = valid ? v : -INFINITY;
+        s[t][e] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, SYN_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, SYN_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing seen yet: every weight below is zero
+    const float alpha = __expf(m - m_use);
+    float sum = 0.f;
+    bf16x4 hi[4], lw[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p = __expf(s[t][e] - m_use);      // exp(-inf) = 0 for what is hidden
+        sum += p;
+        const bf16 h = (bf16)p;
+        hi[t][e] = h;
+        lw[t][e] = (bf16)(p - (float)h);
+      }
+    sum += __shfl_xor(sum, 16, SYN_WAVE);
+    sum += __shfl_xor(sum, 32, SYN_WAVE);
+    l = l * alpha + sum;
+    m = m_new;
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      // k index 8 g + e stands for key 32 pr + 4 g + e, 8 g + 4 + e for key 32 pr + 16 + 4 g + e: both operands agree
+      const bf16x8 b_hi = awp_join(hi[2 * pr], hi[2 * pr + 1]), b_lo = awp_join(lw[2 * pr], lw[2 * pr + 1]);
+#pragma unroll
+      for (int j = 0; j < AWP_TILES; ++j) {
+        if (j < vt) {
+          const bf16* vrow = vpage + (size_t)(16 * j + i) * SYN_PAGE + 32 * pr + 4 * g;
+          const bf16x8 a = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
+          if (pr == 0) O[j] *= alpha;
+          O[j] = awp_mfma32(a, b_hi, O[j]);
+          O[j] = awp_mfma32(a, b_lo, O[j]);
+        }
+      }
+    }
+  }
+  if (!q_ok) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const size_t tok = (size_t)(start + my_n);
+#pragma unroll
+  for (int j = 0; j < AWP_TILES; ++j) {
+    if (j < vt) {
+      const int col = head * vdim + 16 * j + 4 * g;
+      bf16x4 o4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = O[j][e] * inv;
+        if (gate) {
+          const float z = gate[tok * gate_stride + col + e] + (gate_bias ? gate_bias[col + e] : 0.f);
+          v *= 1.f / (1.f + __expf(-z));
+        }
+        o4[e] = (bf16)v;
+      }
+      *(bf16x4*)(out + tok * nh * vdim + col) = o4;
+    }
+  }
+}
+
+// Prompts (and any step that is not single tokens only) in bf16: seq_start [n_seqs + 1] offsets of the sequences' new
+// tokens in q, seq_past [n_seqs] tokens cached before.  Head sizes that are multiples of 16 up to 128.
+SYN_EXPORT int syn_window_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages,
+                                                 const int* page_table, int table_stride, const int* seq_start,
+                                                 const int* seq_past, int n_seqs, int n_tokens, const float* gate,
+                                                 int gate_stride, const float* gate_bias, void* out, float scale, int nh,
+                                                 int nkv, int dim, int vdim, const float* slopes, const float* r1,
+                                                 const float* r2, float softcap, int window, int keep_first, int sink_one,
+                                                 hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && n_seqs > 0 && nh > 0 && nkv > 0, "window_attention_prefill: empty input");
+  SYN_CHECK(nh % nkv == 0, "window_attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
+  SYN_CHECK(dim % 16 == 0 && vdim % 16 == 0 && dim >= 16 && vdim >= 16 && dim <= 16 * AWP_TILES && vdim <= 16 * AWP_TILES,
+            "window_attention_prefill: head sizes %d and %d (multiples of 16 up to %d)", dim, vdim, 16 * AWP_TILES);
+  SYN_CHECK(softcap >= 0.f && window >= 0 && keep_first >= 0, "window_attention_prefill: soft cap %g, window %d, kept %d",
+            (double)softcap, window, keep_first);
+  SYN_CHECK((r1 == nullptr) == (r2 == nullptr), "window_attention_prefill: r1 and r2 come together");
+  SYN_CHECK(gate == nullptr || (gate_stride >= nh * vdim && gate_stride % 4 == 0 && (uintptr_t)gate % 16 == 0),
+            "window_attention_prefill: gate rows of %d values", gate_stride);
+  SYN_CHECK((uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 && (uintptr_t)out % 8 == 0,
+            "window_attention_prefill: operands are not aligned");
+  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one};
+  const dim3 grid((n_tokens + 63) / 64 + n_seqs, nh);      // at most this many tiles of 64 queries; the rest leave at once
+  if (dim % 32 == 0)
+    window_prefill_bf16_kernel<true><<<grid, 256, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
+        gate, gate_stride, gate_bias, (bf16*)out, scale, nh, nkv, dim, vdim, terms);
+  else
+    window_prefill_bf16_kernel<false><<<grid, 256, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
+        gate, gate_stride, gate_bias, (bf16*)out, scale, nh, nkv, dim, vdim, terms);
+  SYN_LAUNCH_CHECK("window_attention_prefill");
   return 0;
 }

@@ -36,6 +36,7 @@ matrix_memory_scan_kernel(const float* __restrict__ proj, int width, const float
   const int v = vt * MM_VT + lane;
   const bool v_ok = v < vdim;
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  if (t0 >= t1) return;     // a sequence without tokens in this step (the spare ones of a padded step): nothing moves
   const int slot = seq_slot[b];
   const size_t per_head = (size_t)dim * vdim + dim + 1;
   float* st = state + ((size_t)(slot < 0 ? spare_row : slot) * H + h) * per_head;

@@ -855,6 +855,52 @@ def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, sca
           1 if sink_one else 0, _stream())
 
 
+WINDOW_PREFILL_MAX_DIM = 128
+
+
+def window_prefill_takes(dim, vdim) -> bool:
+    """Whether the bf16 prompt kernel on the matrix cores takes these head sizes (multiples of 16 up to 128)."""
+    return dim % 16 == 0 and vdim % 16 == 0 and 16 <= dim <= WINDOW_PREFILL_MAX_DIM and 16 <= vdim <= WINDOW_PREFILL_MAX_DIM
+
+
+def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, n_heads, n_kv_heads,
+                                  dim, vdim, window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None,
+                                  softcap=0.0, gate=None, gate_bias=None):
+    """window_attention for the new tokens of each sequence of a step in bf16, on the matrix cores: seq_start [B + 1]
+    offsets of the sequences' new tokens in q, seq_past [B] tokens cached before (the pages already hold the new
+    ones).  Scores and weights are 32-bit; a weight meets V as two bf16 numbers (16 bits of mantissa)."""
+    nh, nkv = n_heads, n_kv_heads
+    if not window_prefill_takes(dim, vdim):
+        raise KernelError(f"window_attention_prefill: head sizes {dim} and {vdim} (multiples of 16 up to {WINDOW_PREFILL_MAX_DIM})")
+    _need(q, "window_attention_prefill.q", _BF16, (None, nh * dim))
+    N = q.shape[0]
+    _check_window_pages(k_pages, v_pages, _BF16, nkv, dim, vdim, "window_attention_prefill")
+    _need(page_table, "window_attention_prefill.page_table", _I32, (None, None))
+    _need(seq_start, "window_attention_prefill.seq_start", _I32, (None,))
+    B = seq_start.shape[0] - 1
+    _need(seq_past, "window_attention_prefill.seq_past", _I32, (B,))
+    if page_table.shape[0] < B:
+        raise KernelError(f"window_attention_prefill: page table has {page_table.shape[0]} rows for {B} sequences")
+    _need(out, "window_attention_prefill.out", _BF16, (N, nh * vdim))
+    r1 = r2 = None
+    if log_bias is not None:
+        r1, r2 = log_bias
+        _need(r1, "window_attention_prefill.r1", _F32, (nh,))
+        _need(r2, "window_attention_prefill.r2", _F32, (nh,))
+    if slopes is not None:
+        _need(slopes, "window_attention_prefill.slopes", _F32, (nh,))
+    gate_stride = 0
+    if gate is not None:
+        gate_stride = _float_rows_view(gate, "window_attention_prefill.gate", N, nh * vdim)
+        if gate_bias is not None:
+            _need(gate_bias, "window_attention_prefill.gate_bias", _F32, (nh * vdim,))
+    _call(load_library("core"), "syn_window_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages),
+          _ptr(page_table), page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(gate), gate_stride,
+          _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), nh, nkv, dim, vdim,
+          _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
+          1 if sink_one else 0, _stream())
+
+
 def _float_rows_view(t, name, n_rows, n_cols):
     """A float tensor [n_rows, >= n_cols] whose rows may be pieces of longer rows (columns of a fused projection):
     returns the row stride in elements."""

@@ -19,7 +19,7 @@ from .mixer import Mixer, _projection
 
 class MatrixMemory(Mixer):
     takes_scaled_rows = False
-    capturable = False      # (its steps are launched one by one)
+    capturable = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "i": "i", "f": "f", "bias": ".b"}
 

@@ -198,7 +198,7 @@ class GatedWindowAttention(Mixer):
     Tensor names: prefix + "q", "k", "v", "o" (+ ".b" for their biases), "q.norm", "k.norm", "g"; `names` renames them.
     """
     takes_scaled_rows = False
-    capturable = False      # (its steps are launched one by one)
+    capturable = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": ".b"}
 
@@ -281,9 +281,16 @@ class GatedWindowAttention(Mixer):
                           write_kv=owner)
         o = torch.empty((N, self.nh * self.vdim), dtype=act, device=h.device)
         gate = proj[:, (self.nh + self.nkv) * self.dim + self.nkv * self.vdim:] if self.gate else None
-        ops.window_attention(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, self.nh,
-                             self.nkv, self.dim, self.vdim, window=self.window or 0, keep_first=self.keep_first,
-                             sink_one=self.sink_one, gate=gate, **self._score_terms(h.device))
+        how = dict(window=self.window or 0, keep_first=self.keep_first, sink_one=self.sink_one, gate=gate,
+                   **self._score_terms(h.device))
+        if act == torch.bfloat16 and not ctx.one_token_each and ops.window_prefill_takes(self.dim, self.vdim):
+            # prompts in bf16: tiles of queries on the matrix cores
+            ops.window_attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
+                                              self.scale, self.nh, self.nkv, self.dim, self.vdim, **how)
+        else:
+            # 32-bit, single tokens, and head sizes that the tiles do not take: a wave (or eight) for each (token, head)
+            ops.window_attention(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, self.nh,
+                                 self.nkv, self.dim, self.vdim, **how)
         y = linear_for_sum(o, self.w_o)
         return WeightedDeltas([(y, 1.0, self.b_o)]) if self.b_o is not None else y
 

@@ -55,7 +55,7 @@ def test_the_model_declares_its_tensors_and_cache_needs():
     needs = model.cache_needs()
     assert needs[0] == (KvNeed(2, 16, 20, v_dim=24, keep_first=3), StateNeed((2, 8 * 16 + 8 + 1)))
     assert needs[1] == (KvNeed(1, 32, 70, v_dim=16, keep_first=0), StateNeed((1, 24 * 40 + 24 + 1)))
-    assert model.streams == 2 and not model.capturable()
+    assert model.streams == 2 and model.capturable()
 
 
 def test_a_cache_layer_may_hold_keys_and_a_state():

@@ -130,6 +130,52 @@ def test_window_attention_sees_exactly_its_keys(window, keep_first, dtype):
     assert float((out.cpu().double() - plain).abs().max()) < tol
 
 
+@pytest.mark.parametrize("D,E,window,keep_first", [(32, 16, 96, 6), (48, 48, 64, 0), (16, 80, 65, 70), (128, 128, 7, 1),
+                                                   (64, 32, 0, 0)])
+def test_window_attention_for_prompts_on_the_matrix_cores(D, E, window, keep_first):
+    """The bf16 prompt kernel against the plain attention, with the peaked scores of the test above: three sequences of
+    unequal lengths in one call, two of which continue from keys that an earlier portion left (the tiles begin inside
+    a page, and their windows reach back into the old keys), and a sequence of one token."""
+    from synaptix_amd.kernels import ops
+    H, G = 4, 2
+    g = torch.Generator().manual_seed(D + E + window)
+    lens, pasts = [150, 1, 77, 203], [0, 0, 130, 61]
+    r1, r2 = torch.tensor([0.3, 0.0, 1.0, 0.5], dtype=P.F64), torch.tensor([0.5, 2.0, 0.05, 1.0], dtype=P.F64)
+    total = [n + p for n, p in zip(lens, pasts)]
+    n_pages = [-(-t // 64) for t in total]
+    kp = torch.full((sum(n_pages) + 1, G, 64, D), 50.0)
+    vp = torch.full((sum(n_pages) + 1, G, E, 64), 50.0)
+    table = torch.zeros((len(lens), max(n_pages)), dtype=torch.int32)
+    order = (torch.randperm(sum(n_pages), generator=g) + 1).tolist()
+    qs, wants, gates = [], [], []
+    for b, T in enumerate(total):
+        kind = torch.randint(0, 4, (T,), generator=g)
+        k = 0.01 * torch.randn(T, G, D, generator=g, dtype=P.F64)
+        k[torch.arange(T), :, kind] += 1.0
+        q = torch.zeros(T, H, D, dtype=P.F64)
+        q[torch.arange(T), :, kind] = 6.0
+        v = torch.randn(T, G, E, generator=g, dtype=P.F64)
+        q, k, v = (t.to(torch.bfloat16).double() for t in (q, k, v))
+        gate = torch.randn(T, H * E, generator=g, dtype=P.F64)
+        want = P.window_attention(q, k, v, 1.5, window or None, keep_first, r1, r2).reshape(T, H * E) * torch.sigmoid(gate)
+        for pg in range(n_pages[b]):
+            table[b, pg] = order.pop()
+        for t in range(T):
+            kp[table[b, t // 64], :, t % 64] = k[t].float()
+            vp[table[b, t // 64], :, :, t % 64] = v[t].float()
+        qs.append(q[pasts[b]:].reshape(lens[b], H * D))
+        wants.append(want[pasts[b]:])
+        gates.append(gate[pasts[b]:])
+    start = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    out = torch.empty((sum(lens), H * E), dtype=torch.bfloat16, device=DEV)
+    ops.window_attention_prefill_bf16(dev(torch.cat(qs), torch.bfloat16), dev(kp, torch.bfloat16), dev(vp, torch.bfloat16),
+                                      table.to(DEV), start, torch.tensor(pasts, dtype=torch.int32, device=DEV), out, 1.5,
+                                      H, G, D, E, window=window, keep_first=keep_first, sink_one=True,
+                                      log_bias=(dev(r1), dev(r2)), gate=dev(torch.cat(gates)))
+    err = (out.cpu().double() - torch.cat(wants)).abs()
+    assert float(err.max()) < 1.5e-2, f"max err {float(err.max())} at row {int(err.max(1).values.argmax())}"
+
+
 def test_window_intake_norms_q_and_k_and_writes_the_pages():
     from synaptix_amd.kernels import ops
     g = torch.Generator().manual_seed(5)
@@ -349,3 +395,47 @@ def test_greedy_generation_through_the_pipeline(dtype):
                 assert tok == best or float(row[best] - row[tok]) < 1e-4
             else:
                 assert tok == best or float(row[best] - row[tok]) < 0.05 * float(row.abs().max())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["P", "R"])
+def test_decode_steps_replayed_from_a_graph(name, dtype):
+    """Captured decode steps (three rows wide in a graph of four: one row is padding) with eager work of other
+    sequences between the replays; every replay against the plain model, and the states of the sequences that a
+    capture ran twice must be where a single step leaves them."""
+    eng = engine(name, dtype, max_tokens=64 * 12)
+    assert eng.graph_ok
+    reqs = [tokens_for(name, n, 40 + n) for n in (90, 20, 140)]
+    other = tokens_for(name, 60, 4)
+    want = [plain_logits(name, r) for r in reqs]
+    heads = [len(r) - 12 for r in reqs]
+    slots = [eng.acquire() for _ in reqs]
+    eng.step([(s, r[:h]) for s, r, h in zip(slots, reqs, heads)], want=None)
+    runner = eng.decode_runner(3, 256)
+    assert runner.rows == 4
+    extra = eng.acquire()
+    for i in range(12):
+        _, lg = runner.step(slots, [r[h + i] for r, h in zip(reqs, heads)])
+        for j in range(3):
+            assert_logits_close(lg[j:j + 1].clone(), want[j][heads[j] + i:heads[j] + i + 1], dtype,
+                                f"{name} {dtype} replay {i} row {j}", sharp=True)
+        got = eng.step([(extra, other[5 * i:5 * i + 5])], want="last")        # an eager prompt portion in between
+        assert_logits_close(got, plain_logits(name, other)[5 * i + 4:5 * i + 5], dtype, f"{name} {dtype} eager between replays",
+                            sharp=True)
+    eng.cache.check()
+
+
+def test_short_prompt_steps_replayed_from_a_graph():
+    """bfloat16 prompt steps of a few tokens go through captured graphs with padding rows (an extra sequence on the
+    spare page and the spare state row); portions of a prompt one after another, each from what the last one left."""
+    name = "R"
+    eng = engine(name, "bfloat16")
+    assert eng.graph_ok and eng.prompt_graphs
+    toks = tokens_for(name, 120, 8)
+    want = plain_logits(name, toks)
+    s, at = eng.acquire(), 0
+    for n in (10, 10, 30, 10, 40, 20):
+        got = eng.step([(s, toks[at:at + n])], want="last")
+        at += n
+        assert_logits_close(got, want[at - 1:at], "bfloat16", f"prompt portion ending at {at} through a graph", sharp=True)
+    assert any(k[0] == "prompt" for k in eng._runners), "no prompt step was replayed from a graph"
