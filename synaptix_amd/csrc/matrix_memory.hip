@@ -120,11 +120,220 @@ matrix_memory_scan_kernel(const float* __restrict__ proj, int width, const float
   }
 }
 
+// The same cell for prompts, a chunk of MMC_L tokens at a time.  Inside a chunk, with b_t the sum of f from the chunk's
+// first token to t, m_0, S_0, n_0 the state before the chunk:
+//   m_t = b_t + max(m_0, max_(s <= t) (i_s - b_s))                                (the recurrence of m, unrolled)
+//   A[t][s] = (q_t . k_s) exp(b_t - b_s + i_s - m_t) for s <= t, g_t = exp(b_t + m_0 - m_t)
+//   S_t^T q_t = sum_s A[t][s] v_s + g_t S_0^T q_t,      n_t . q_t = sum_s A[t][s] + g_t n_0 . q_t
+//   S_L = exp(b_L + m_0 - m_L) S_0 + sum_s exp(b_L - b_s + i_s - m_L) k_s v_s^T   (n likewise)
+// Every exponent is at most 0, as in the step-by-step form; all sums are 32-bit FMA.  b_t and m_t grow with the chunk
+// (up to 32 times a log gate), and the exponents are small differences of them: they are kept in 64-bit inside the
+// chunk, so that an exponent is as exact as the step-by-step form's, whose f + m - m' never leaves the size of one gate.
+// A workgroup keeps its 64 columns of S in registers between chunks (rows w, w + 4, ... in wave w, as above) and
+// stages q, k, v, A and S_0 in LDS.
+#define MMC_L 32
+
+__host__ __device__ inline size_t mmc_lds_floats(int dim) {
+  return (size_t)2 * MMC_L * (dim + 1) + MMC_L * MM_VT + MMC_L * (MMC_L + 1) + (size_t)dim * MM_VT + dim + 8 * MMC_L + 4;
+}
+
+template <int DPT>
+__global__ void __launch_bounds__(MM_DG * SYN_WAVE)
+matrix_memory_chunk_kernel(const float* __restrict__ proj, int width, const float* __restrict__ i_bias,
+                           const float* __restrict__ f_bias, float cap, float q_scale, float* __restrict__ state,
+                           int spare_row, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+                           float* __restrict__ out, int H, int dim, int vdim) {
+  extern __shared__ float lds[];
+  constexpr int L = MMC_L;
+  const int DP = dim + 1;
+  double* bs = (double*)lds;             // [L] b_t
+  double* ms = bs + L;                   // [L] m_t
+  float* qs = (float*)(ms + L);          // [L][DP]  q, scaled
+  float* ks = qs + L * DP;               // [L][DP]
+  float* vs = ks + L * DP;               // [L][64]  this workgroup's columns of v
+  float* As = vs + L * MM_VT;            // [L][L + 1]
+  float* Cs = As + L * (L + 1);          // [dim][64]  S before the chunk
+  float* ns = Cs + (size_t)dim * MM_VT;  // [dim]      n before the chunk
+  float* ig_s = ns + dim;                // [L] i_t
+  float* gq = ig_s + L;                  // [L] g_t
+  float* ws = gq + L;                    // [L] exp(b_L - b_s + i_s - m_L)
+  float* rs = ws + L;                    // [L] n_t . q_t
+  float* sc = rs + L;                    // [0] exp(b_L + m_0 - m_L), [1] m_L
+  const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, tid = threadIdx.x;
+  const int v = vt * MM_VT + lane;
+  const bool v_ok = v < vdim;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  if (t0 >= t1) return;
+  const int slot = seq_slot[b];
+  const size_t per_head = (size_t)dim * vdim + dim + 1;
+  float* st = state + ((size_t)(slot < 0 ? spare_row : slot) * H + h) * per_head;
+  const int q_col = h * dim, k_col = H * dim + h * dim, v_col = 2 * H * dim + h * vdim;
+  const int i_col = 2 * H * dim + 2 * H * vdim + h, f_col = i_col + H;
+  const float bi = i_bias ? i_bias[h] : 0.f, bf = f_bias ? f_bias[h] : 0.f;
+
+  float S[DPT];
+#pragma unroll
+  for (int j = 0; j < DPT; ++j) {
+    const int d = wave + MM_DG * j;
+    S[j] = (d < dim && v_ok) ? st[(size_t)d * vdim + v] : 0.f;
+  }
+  const int dn = wave + MM_DG * lane;
+  float n = dn < dim ? st[(size_t)dim * vdim + dn] : 0.f;
+  float m = st[(size_t)dim * vdim + dim];
+
+  for (int c0 = t0; c0 < t1; c0 += L) {
+    const int nc = min(L, t1 - c0);
+    __syncthreads();
+    for (int idx = tid; idx < L * dim; idx += blockDim.x) {
+      const int t = idx / dim, d = idx % dim;
+      const float* row = proj + (size_t)(c0 + min(t, nc - 1)) * width;
+      qs[t * DP + d] = t < nc ? row[q_col + d] * q_scale : 0.f;
+      ks[t * DP + d] = t < nc ? row[k_col + d] : 0.f;
+    }
+    for (int idx = tid; idx < L * MM_VT; idx += blockDim.x) {
+      const int t = idx / MM_VT, c = idx % MM_VT;
+      vs[idx] = (t < nc && vt * MM_VT + c < vdim) ? proj[(size_t)(c0 + t) * width + v_col + vt * MM_VT + c] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) {
+      const int d = wave + MM_DG * j;
+      if (d < dim) Cs[(size_t)d * MM_VT + lane] = S[j];
+    }
+    if (dn < dim) ns[dn] = n;
+    if (wave == 0) {
+      // the gates of the chunk's tokens, one a lane; sums and maxima along the lanes
+      float ig = -INFINITY, fg = 0.f;
+      if (lane < nc) {
+        const float* row = proj + (size_t)(c0 + lane) * width;
+        const float ri = row[i_col] + bi, rf = row[f_col] + bf;
+        ig = cap > 0.f ? cap * tanhf(ri / cap) : ri;
+        fg = log_sigmoid(cap > 0.f ? cap * tanhf(rf / cap) : rf);
+      }
+      double bsum = fg;
+#pragma unroll
+      for (int off = 1; off < L; off <<= 1) {
+        const double x = __shfl_up(bsum, off, SYN_WAVE);
+        if (lane >= off) bsum += x;
+      }
+      double pm = lane < nc ? (double)ig - bsum : -INFINITY;
+#pragma unroll
+      for (int off = 1; off < L; off <<= 1) {
+        const double x = __shfl_up(pm, off, SYN_WAVE);
+        if (lane >= off) pm = fmax(pm, x);
+      }
+      const double mt = bsum + fmax((double)m, pm);
+      const double bL = __shfl(bsum, nc - 1, SYN_WAVE), mL = __shfl(mt, nc - 1, SYN_WAVE);
+      if (lane < L) {
+        bs[lane] = bsum, ig_s[lane] = ig, ms[lane] = mt;
+        gq[lane] = expf((float)(bsum + m - mt));
+        ws[lane] = lane < nc ? expf((float)(bL - bsum + ig - mL)) : 0.f;
+      }
+      if (lane == 0) sc[0] = expf((float)(bL + m - mL)), sc[1] = (float)mL;
+    }
+    __syncthreads();
+    {
+      // A[t][s]: thread tid takes t = tid / 8 and the four s = 4 (tid % 8) ..
+      const int t = tid / 8, s0 = 4 * (tid % 8);
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      if (s0 <= t) {
+        const float* qr = qs + t * DP;
+        const float* kr = ks + s0 * DP;
+        for (int d = 0; d < dim; ++d) {
+          const float qv = qr[d];
+          a0 = fmaf(qv, kr[d], a0), a1 = fmaf(qv, kr[DP + d], a1);
+          a2 = fmaf(qv, kr[2 * DP + d], a2), a3 = fmaf(qv, kr[3 * DP + d], a3);
+        }
+      }
+      const double btm = bs[t] - ms[t];
+      float* ar = As + t * (L + 1) + s0;
+      const bool row_ok = t < nc;
+      ar[0] = (row_ok && s0 <= t) ? a0 * expf((float)(btm - bs[s0] + ig_s[s0])) : 0.f;
+      ar[1] = (row_ok && s0 + 1 <= t) ? a1 * expf((float)(btm - bs[s0 + 1] + ig_s[s0 + 1])) : 0.f;
+      ar[2] = (row_ok && s0 + 2 <= t) ? a2 * expf((float)(btm - bs[s0 + 2] + ig_s[s0 + 2])) : 0.f;
+      ar[3] = (row_ok && s0 + 3 <= t) ? a3 * expf((float)(btm - bs[s0 + 3] + ig_s[s0 + 3])) : 0.f;
+    }
+    __syncthreads();
+    // wave w takes the tokens 8 w .. 8 w + 7: their n . q first, then this lane's column of S^T q
+    constexpr int R = L / MM_DG;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int t = wave * R + r;
+      float part = lane < L ? As[t * (L + 1) + lane] : 0.f;
+      float nq0 = 0.f;
+      for (int d = lane; d < dim; d += SYN_WAVE) nq0 = fmaf(ns[d], qs[t * DP + d], nq0);
+      part = wave_sum(part + gq[t] * nq0);
+      if (lane == 0) rs[t] = part;
+    }
+    float acc[R], acc0[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f, acc0[r] = 0.f;
+    for (int s = 0; s < nc; ++s) {
+      const float vv = vs[s * MM_VT + lane];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = fmaf(As[(wave * R + r) * (L + 1) + s], vv, acc[r]);
+    }
+    for (int d = 0; d < dim; ++d) {
+      const float cv = Cs[(size_t)d * MM_VT + lane];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc0[r] = fmaf(qs[(wave * R + r) * DP + d], cv, acc0[r]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // rs[t] of this wave's tokens, written by its lane 0
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int t = wave * R + r;
+      if (t < nc && v_ok) {
+        const float den = fmaxf(fabsf(rs[t]), expf(-(float)ms[t])) + 1e-6f;
+        out[(size_t)(c0 + t) * H * vdim + (size_t)h * vdim + v] = (acc[r] + gq[t] * acc0[r]) / den;
+      }
+    }
+    // the state behind the chunk
+    const float G = sc[0];
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) S[j] *= G;
+    for (int s = 0; s < nc; ++s) {
+      const float wv = ws[s] * vs[s * MM_VT + lane];
+#pragma unroll
+      for (int j = 0; j < DPT; ++j) {
+        const int d = wave + MM_DG * j;
+        if (d < dim) S[j] = fmaf(ks[s * DP + d], wv, S[j]);
+      }
+    }
+    if (dn < dim) {
+      float nn = G * n;
+      for (int s = 0; s < nc; ++s) nn = fmaf(ws[s], ks[s * DP + dn], nn);
+      n = nn;
+    }
+    m = sc[1];
+  }
+#pragma unroll
+  for (int j = 0; j < DPT; ++j) {
+    const int d = wave + MM_DG * j;
+    if (d < dim && v_ok) st[(size_t)d * vdim + v] = S[j];
+  }
+  if (vt == 0) {
+    if (dn < dim) st[(size_t)dim * vdim + dn] = n;
+    if (threadIdx.x == 0) st[(size_t)dim * vdim + dim] = m;
+  }
+}
+
+template <int DPT>
+static hipError_t raise_chunk_lds() {
+  static OncePerDevice once;
+  return once_per_device(once, [] {
+    return hipFuncSetAttribute((const void*)matrix_memory_chunk_kernel<DPT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)(mmc_lds_floats(4 * DPT) * sizeof(float)));
+  });
+}
+
 // out [N][H * vdim] float: o_t of every token, before the heads' norm
+// chunked: 0 = token by token (single tokens), 1 = in chunks (prompts)
 SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float* i_bias, const float* f_bias, float cap,
                                       float q_scale, float* state, int state_rows, const int* seq_start,
                                       const int* seq_slot, int n_seqs, float* out, int H, int dim, int vdim,
-                                      hipStream_t stream) {
+                                      int chunked, hipStream_t stream) {
   SYN_CHECK(n_seqs > 0 && H > 0, "matrix_memory_scan: empty input");
   SYN_CHECK(dim > 0 && dim <= MM_MAX_DIM && vdim > 0, "matrix_memory_scan: sizes %d x %d (keys up to %d)", dim, vdim,
             MM_MAX_DIM);
@@ -133,6 +342,24 @@ SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float*
   SYN_CHECK(state_rows >= 1, "matrix_memory_scan: no state rows");
   const dim3 grid(n_seqs, H, (vdim + MM_VT - 1) / MM_VT);
   const int dpt = (dim + MM_DG - 1) / MM_DG;
+  if (chunked) {
+    const size_t lds = mmc_lds_floats(dim) * sizeof(float);
+#define SYN_MMC(D)                                                                                                      \
+  do {                                                                                                                  \
+    const hipError_t e = raise_chunk_lds<D>();                                                                           \
+    SYN_CHECK(e == hipSuccess, "matrix_memory_scan: the chunk kernel's LDS: %s", hipGetErrorString(e));                  \
+    matrix_memory_chunk_kernel<D><<<grid, MM_DG * SYN_WAVE, lds, stream>>>(proj, width, i_bias, f_bias, cap, q_scale,   \
+                                                                           state, state_rows - 1, seq_start, seq_slot, \
+                                                                           out, H, dim, vdim);                          \
+  } while (0)
+    if (dpt <= 8) SYN_MMC(8);
+    else if (dpt <= 16) SYN_MMC(16);
+    else if (dpt <= 32) SYN_MMC(32);
+    else SYN_MMC(64);
+#undef SYN_MMC
+    SYN_LAUNCH_CHECK("matrix_memory_scan (chunks)");
+    return 0;
+  }
 #define SYN_MM(D)                                                                                                   \
   matrix_memory_scan_kernel<D><<<grid, MM_DG * SYN_WAVE, 0, stream>>>(proj, width, i_bias, f_bias, cap, q_scale, state, \
                                                                       state_rows - 1, seq_start, seq_slot, out, H, dim, vdim)

@@ -921,10 +921,12 @@ def matrix_memory_state_size(dim, vdim) -> int:
     return dim * vdim + dim + 1
 
 
-def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim,
+                       chunked=False):
     """The cell of csrc/matrix_memory.hip over the new tokens of every sequence of the step, in order, from and into
     state [rows, H, dim * vdim + dim + 1] float (row = seq_slot[b]; a negative slot takes the last row).
-    proj [N, width] float: [q | k | v | gate | i | f] of the fused projection; out [N, H * vdim] float."""
+    proj [N, width] float: [q | k | v | gate | i | f] of the fused projection; out [N, H * vdim] float.
+    chunked: 32 tokens at a time (prompts) instead of token by token (single tokens); the same sums in another order."""
     H = n_heads
     _need(proj, "matrix_memory_scan.proj", _F32, (None, None))
     N, width = proj.shape
@@ -942,7 +944,7 @@ def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start
     _need(out, "matrix_memory_scan.out", _F32, (N, H * vdim))
     _call(load_library("core"), "syn_matrix_memory_scan", _ptr(proj), width, _ptr(i_bias), _ptr(f_bias),
           ctypes.c_float(float(gate_cap or 0.0)), ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(seq_start),
-          _ptr(seq_slot), B, _ptr(out), H, dim, vdim, _stream())
+          _ptr(seq_slot), B, _ptr(out), H, dim, vdim, 1 if chunked else 0, _stream())
 
 
 def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim):

@@ -204,8 +204,9 @@ def test_window_intake_norms_q_and_k_and_writes_the_pages():
         assert float((vp[page, :, :, pos % 64] - v[n]).abs().max()) < 1e-5
 
 
-@pytest.mark.parametrize("H,D,E,T", [(2, 10, 72, 150), (1, 64, 16, 40), (3, 5, 130, 33)])
-def test_matrix_memory_in_portions_and_slots(H, D, E, T):
+@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("H,D,E,T", [(2, 10, 72, 150), (1, 64, 16, 40), (3, 5, 130, 33), (1, 130, 64, 70)])
+def test_matrix_memory_in_portions_and_slots(H, D, E, T, chunked):
     """Two sequences in one step (their states in rows 2 and 0), then the rest of both in a second step from the
     states the first left; gates drawn wide so that the running maximum moves and old contents decay."""
     from synaptix_amd.kernels import ops
@@ -238,13 +239,15 @@ def test_matrix_memory_in_portions_and_slots(H, D, E, T):
         start = torch.tensor([0, pieces[0].shape[0], proj.shape[0]], dtype=torch.int32, device=DEV)
         slot = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
         out = torch.empty((proj.shape[0], H * E), dtype=torch.float32, device=DEV)
-        ops.matrix_memory_scan(proj, dev(ib), dev(fb), cap, D ** -0.5, state, start, slot, out, H, D, E)
+        ops.matrix_memory_scan(proj, dev(ib), dev(fb), cap, D ** -0.5, state, start, slot, out, H, D, E, chunked=chunked)
         got[2].append(out[:pieces[0].shape[0]])
         got[0].append(out[pieces[0].shape[0]:])
     for s in seqs:
         o = torch.cat(got[s]).cpu().double().view(-1, H, E)
+        # (o is a quotient whose divisor n . q cancels now and then: where it does, a last-bit difference in a sum
+        # is a larger one in o, so the bound on o is wider than the one on the state below)
         scale = float(want[s][0].abs().max())
-        assert float((o - want[s][0]).abs().max()) < 2e-5 * max(1.0, scale)
+        assert float((o - want[s][0]).abs().max()) < 6e-5 * max(1.0, scale)
         C, n, m = want[s][1]
         st = state[s].cpu().double()
         assert float((st[:, :D * E].view(H, D, E) - C).abs().max()) < 2e-5 * max(1.0, float(C.abs().max()))
