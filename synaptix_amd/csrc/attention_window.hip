@@ -110,6 +110,18 @@ __device__ __forceinline__ float window_score(float dot, float scale, const Wind
   return s;
 }
 
+// eight consecutive values of a cache row as floats: one 16-byte load in bf16, two in 32-bit
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&o)[8]);
+template <> __device__ __forceinline__ void load8<bf16>(const bf16* p, float (&o)[8]) {
+  const bf16x8 v = *(const bf16x8*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (float)v[e];
+}
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&o)[8]) {
+  const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
+  o[0] = a.x, o[1] = a.y, o[2] = a.z, o[3] = a.w, o[4] = b.x, o[5] = b.y, o[6] = b.z, o[7] = b.w;
+}
+
 // WAVES waves a (token, head): wave w takes every WAVES-th of the visible blocks of 64 keys, and the waves' partial
 // results (maximum, sum, weighted values) are merged through LDS at the end.  One wave is enough where a step has many
 // tokens; single tokens over a long window get eight.
@@ -154,7 +166,16 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     if (valid) {
       const T* kr = k_pages + kbase + (size_t)lane * dim;
       float dot = 0.f;
-      for (int d = 0; d < dim; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
+      if (dim % 8 == 0) {
+        for (int d = 0; d < dim; d += 8) {
+          float kv[8];
+          load8<T>(kr + d, kv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dot = fmaf(qs[d + e], kv[e], dot);
+        }
+      } else {
+        for (int d = 0; d < dim; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
+      }
       s = window_score(dot, scale, terms, slope, r1, r2, pos, key);
     }
     const float m_new = fmaxf(m, wave_max(s));   // every block that is visited holds a visible key
@@ -176,9 +197,14 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
       if (d < vdim) {
         const T* vr = v_pages + vbase + (size_t)d * SYN_PAGE;
         float acc = o[i] * alpha;
-        for (int j = 0; j < SYN_PAGE; ++j) {
-          const float pj = ps[wave][j];
-          if (pj != 0.f) acc = fmaf(pj, to_f32<T>(vr[j]), acc);   // slots past the sequence's end may hold anything
+        for (int j = 0; j < SYN_PAGE; j += 8) {
+          float vv[8];
+          load8<T>(vr + j, vv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float pj = ps[wave][j + e];
+            acc = fmaf(pj, pj != 0.f ? vv[e] : 0.f, acc);   // slots past the sequence's end may hold anything
+          }
         }
         o[i] = acc;
       }
@@ -331,25 +357,59 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
 #pragma unroll
   for (int j = 0; j < AWP_TILES; ++j) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int idx = 0; idx < n_blocks; ++idx) {
-    const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
-    const int page = page_table[(size_t)seq * table_stride + kb];
+  // The K fragments of a page are asked for one page ahead (behind the products that used the last ones), the V
+  // fragments at the top of their page, ahead of the scores and the softmax that hide their way from memory.
+  bf16x8 kf8[4][AWP_TILES / 2];
+  bf16x4 kf4[4][AWP_TILES];
+  auto block_of = [&](int idx) { return idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks); };
+  auto load_k = [&](int page) {
     const bf16* kpage = k_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * dim;
-    const bf16* vpage = v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
-    f32x4 s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
       const bf16* krow = kpage + (size_t)(16 * t + i) * dim;
       if constexpr (X32) {
 #pragma unroll
         for (int c = 0; c < AWP_TILES / 2; ++c)
-          if (c < dim / 32) s[t] = awp_mfma32(*(const bf16x8*)(krow + 32 * c + 8 * g), qf8[c], s[t]);
+          if (c < dim / 32) kf8[t][c] = *(const bf16x8*)(krow + 32 * c + 8 * g);
       } else {
 #pragma unroll
         for (int c = 0; c < AWP_TILES; ++c)
-          if (c < dim / 16) s[t] = awp_mfma16(*(const bf16x4*)(krow + 16 * c + 4 * g), qf4[c], s[t]);
+          if (c < dim / 16) kf4[t][c] = *(const bf16x4*)(krow + 16 * c + 4 * g);
       }
+    }
+  };
+  int page = page_table[(size_t)seq * table_stride + block_of(0)];
+  load_k(page);
+  for (int idx = 0; idx < n_blocks; ++idx) {
+    const int kb = block_of(idx);
+    const bf16* vpage = v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
+    bf16x8 vf[2][AWP_TILES];
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+      for (int j = 0; j < AWP_TILES; ++j)
+        if (j < vt) {
+          // k index 8 g + e stands for key 32 pr + 4 g + e, 8 g + 4 + e for key 32 pr + 16 + 4 g + e (see below)
+          const bf16* vrow = vpage + (size_t)(16 * j + i) * SYN_PAGE + 32 * pr + 4 * g;
+          vf[pr][j] = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
+        }
+    f32x4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (X32) {
+#pragma unroll
+        for (int c = 0; c < AWP_TILES / 2; ++c)
+          if (c < dim / 32) s[t] = awp_mfma32(kf8[t][c], qf8[c], s[t]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < AWP_TILES; ++c)
+          if (c < dim / 16) s[t] = awp_mfma16(kf4[t][c], qf4[c], s[t]);
+      }
+    }
+    if (idx + 1 < n_blocks) {
+      page = page_table[(size_t)seq * table_stride + block_of(idx + 1)];
+      load_k(page);
     }
     // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i)
     float mx = -INFINITY;
@@ -396,11 +456,9 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
 #pragma unroll
       for (int j = 0; j < AWP_TILES; ++j) {
         if (j < vt) {
-          const bf16* vrow = vpage + (size_t)(16 * j + i) * SYN_PAGE + 32 * pr + 4 * g;
-          const bf16x8 a = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
           if (pr == 0) O[j] *= alpha;
-          O[j] = awp_mfma32(a, b_hi, O[j]);
-          O[j] = awp_mfma32(a, b_lo, O[j]);
+          O[j] = awp_mfma32(vf[pr][j], b_hi, O[j]);
+          O[j] = awp_mfma32(vf[pr][j], b_lo, O[j]);
         }
       }
     }

@@ -922,11 +922,13 @@ def matrix_memory_state_size(dim, vdim) -> int:
 
 
 def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim,
-                       chunked=False):
+                       chunked=False, scratch=None):
     """The cell of csrc/matrix_memory.hip over the new tokens of every sequence of the step, in order, from and into
     state [rows, H, dim * vdim + dim + 1] float (row = seq_slot[b]; a negative slot takes the last row).
     proj [N, width] float: [q | k | v | gate | i | f] of the fused projection; out [N, H * vdim] float.
-    chunked: 32 tokens at a time (prompts) instead of token by token (single tokens); the same sums in another order."""
+    chunked: 32 tokens at a time (prompts) instead of token by token (single tokens); the same sums in another order.
+    scratch: with chunked, a function (name, floats) -> float tensor for the chunks' partial states (StepContext.scratch;
+    default: a new tensor)."""
     H = n_heads
     _need(proj, "matrix_memory_scan.proj", _F32, (None, None))
     N, width = proj.shape
@@ -942,9 +944,18 @@ def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start
     B = seq_start.shape[0] - 1
     _need(seq_slot, "matrix_memory_scan.seq_slot", _I32, (B,))
     _need(out, "matrix_memory_scan.out", _F32, (N, H * vdim))
-    _call(load_library("core"), "syn_matrix_memory_scan", _ptr(proj), width, _ptr(i_bias), _ptr(f_bias),
+    lib = load_library("core")
+    work = None
+    if chunked:
+        lib.syn_matrix_memory_chunk_scratch.restype = ctypes.c_long
+        need = lib.syn_matrix_memory_chunk_scratch(N, B, H, dim, vdim)
+        work = scratch("matrix_memory_chunks", need) if scratch is not None else torch.empty(need, dtype=_F32, device=proj.device)
+        _need(work, "matrix_memory_scan.scratch", _F32)
+        if work.numel() < need:
+            raise KernelError(f"matrix_memory_scan: scratch of {work.numel()} floats, {need} are needed")
+    _call(lib, "syn_matrix_memory_scan", _ptr(proj), width, _ptr(i_bias), _ptr(f_bias),
           ctypes.c_float(float(gate_cap or 0.0)), ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(seq_start),
-          _ptr(seq_slot), B, _ptr(out), H, dim, vdim, 1 if chunked else 0, _stream())
+          _ptr(seq_slot), B, _ptr(out), H, dim, vdim, 1 if chunked else 0, N, _ptr(work), _stream())
 
 
 def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim):

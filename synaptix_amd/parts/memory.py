@@ -66,7 +66,8 @@ class MatrixMemory(Mixer):
         proj = linear(h, self.w_in, torch.float32)          # [N, q | k | v | gate | i | f] float
         raw = torch.empty((N, H * self.vdim), dtype=torch.float32, device=h.device)
         ops.matrix_memory_scan(proj, self.i_bias, self.f_bias, self.gate_cap, self.q_scale, cache.state, ctx.seq_start,
-                               ctx.seq_slot, raw, H, self.dim, self.vdim, chunked=not ctx.one_token_each)
+                               ctx.seq_slot, raw, H, self.dim, self.vdim, chunked=not ctx.one_token_each,
+                               scratch=ctx.scratch)
         o = torch.empty((N, H * self.vdim), dtype=h.dtype, device=h.device)
         ops.head_norm_gate(raw, self.gain, self.norm_eps, proj[:, 2 * H * self.dim + H * self.vdim:], o, H, self.vdim)
         return linear_for_sum(o, self.w_o)
