@@ -282,8 +282,9 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
 }
 
 // ---------------------------------------------------------------- prompts in bf16 on the matrix cores
-// One wave for 16 queries of one (sequence, head), four such waves a workgroup, no LDS and no barrier: a wave walks
-// the pages its queries see, 64 keys at a time.  S^T = K Q^T (MFMA 16x16: a lane then holds four keys of ONE query, so
+// One wave for 16 queries of one (sequence, head), four such waves a workgroup: the workgroup walks the pages that its
+// 64 queries see, a page of 64 keys at a time through LDS, and a wave leaves out a page none of whose keys it sees.
+// S^T = K Q^T (MFMA 16x16: a lane then holds four keys of ONE query, so
 // the softmax's statistics are a lane's own plus two exchanges across the lane groups), and the accumulator's layout
 // is the B operand of O^T += V^T P^T, whose A operand are 8-byte pieces of the V page's rows.  The weights meet V as
 // two bf16 numbers each (the weight rounded, and what the rounding left), so that they count with 16 bits of mantissa
@@ -304,6 +305,9 @@ __device__ __forceinline__ bf16x8 awp_join(bf16x4 lo, bf16x4 hi) {
   return r;
 }
 
+#define AWP_KPAD 8      // bf16 values behind a K row in LDS, so that the 16 rows of a fragment fall into different banks
+#define AWP_VPAD 4      // the same for a V row (64 tokens)
+
 template <bool X32>
 __global__ void __launch_bounds__(256)
 window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
@@ -311,7 +315,9 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
                            const int* __restrict__ seq_past, int n_seqs, const float* __restrict__ gate, int gate_stride,
                            const float* __restrict__ gate_bias, bf16* __restrict__ out, float scale, int nh, int nkv,
                            int dim, int vdim, WindowTerms terms) {
-  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, g = lane / 16;
+  __shared__ __attribute__((aligned(16))) bf16 Ks[SYN_PAGE * (16 * AWP_TILES + AWP_KPAD)];
+  __shared__ __attribute__((aligned(16))) bf16 Vs[16 * AWP_TILES * (SYN_PAGE + AWP_VPAD)];
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE, i = lane % 16, g = lane / 16;
   int bt = blockIdx.x, seq = -1, n_new = 0, start = 0;
   for (int b = 0; b < n_seqs; ++b) {
     const int s0 = seq_start[b], n = seq_start[b + 1] - s0, tiles = (n + 63) / 64;
@@ -321,15 +327,15 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
     }
     bt -= tiles;
   }
-  if (seq < 0) return;
-  const int n0 = bt * 64 + wave * 16;
-  if (n0 >= n_new) return;
+  if (seq < 0) return;                              // (the whole workgroup: no barrier has been reached yet)
+  const int nb = bt * 64, n0 = nb + wave * 16;       // the workgroup's and this wave's first query
+  const bool wave_on = n0 < n_new;                   // a wave without queries still helps to stage the pages
   const int head = blockIdx.y, kvh = head / (nh / nkv);
   const int past = seq_past[seq];
   const bool q_ok = n0 + i < n_new;
   const int my_n = min(n0 + i, n_new - 1);       // (rows beyond the sequence's tokens repeat its last one and are not stored)
   const int qpos = past + my_n;
-  const int vt = vdim / 16;
+  const int vt = vdim / 16, KLD = dim + AWP_KPAD, VLD = SYN_PAGE + AWP_VPAD;
   const bf16* qrow = q + ((size_t)(start + my_n) * nh + head) * dim;
   bf16x8 qf8[AWP_TILES / 2];
   bf16x4 qf4[AWP_TILES];
@@ -344,8 +350,11 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
   }
   const int W = terms.window;
   const int lo_q = W > 0 ? max(0, qpos - W + 1) : 0;                          // this lane's query
-  const int lo_first = W > 0 ? max(0, past + n0 - W + 1) : 0;                 // the tile's first query
-  const int kmax = past + min(n0 + 15, n_new - 1);
+  const int lo_wave = W > 0 ? max(0, past + n0 - W + 1) : 0;                  // this wave's first query
+  const int kmax_wave = past + min(n0 + 15, n_new - 1);
+  // the pages that the workgroup's 64 queries see together
+  const int lo_first = W > 0 ? max(0, past + nb - W + 1) : 0;
+  const int kmax = past + min(nb + 63, n_new - 1);
   const int kept = min(terms.keep_first, lo_first);
   const int n_kept_blocks = kept > 0 ? (kept - 1) / SYN_PAGE + 1 : 0;
   const int first_window_block = max(lo_first / SYN_PAGE, n_kept_blocks);
@@ -357,59 +366,61 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
 #pragma unroll
   for (int j = 0; j < AWP_TILES; ++j) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The K fragments of a page are asked for one page ahead (behind the products that used the last ones), the V
-  // fragments at the top of their page, ahead of the scores and the softmax that hide their way from memory.
-  bf16x8 kf8[4][AWP_TILES / 2];
-  bf16x4 kf4[4][AWP_TILES];
+  // A page's K and V go from memory to registers in whole 16-byte pieces, a row piece after another (every thread
+  // up to four of each), one page ahead of the page that is being multiplied, and from there into LDS.
+  constexpr int PIECES = 16 * AWP_TILES * SYN_PAGE / 8 / 256;      // 4
+  uint4 kreg[PIECES], vreg[PIECES];
   auto block_of = [&](int idx) { return idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks); };
-  auto load_k = [&](int page) {
-    const bf16* kpage = k_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * dim;
+  auto fetch = [&](int idx) {
+    const int page = page_table[(size_t)seq * table_stride + block_of(idx)];
+    const uint4* kp = (const uint4*)(k_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * dim);
+    const uint4* vp = (const uint4*)(v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const bf16* krow = kpage + (size_t)(16 * t + i) * dim;
-      if constexpr (X32) {
+    for (int r = 0; r < PIECES; ++r) {
+      const int it = tid + 256 * r;
+      if (it < SYN_PAGE * dim / 8) kreg[r] = kp[it];
+      if (it < SYN_PAGE * vdim / 8) vreg[r] = vp[it];
+    }
+  };
+  auto stage = [&]() {
 #pragma unroll
-        for (int c = 0; c < AWP_TILES / 2; ++c)
-          if (c < dim / 32) kf8[t][c] = *(const bf16x8*)(krow + 32 * c + 8 * g);
-      } else {
-#pragma unroll
-        for (int c = 0; c < AWP_TILES; ++c)
-          if (c < dim / 16) kf4[t][c] = *(const bf16x4*)(krow + 16 * c + 4 * g);
+    for (int r = 0; r < PIECES; ++r) {
+      const int it = tid + 256 * r;
+      if (it < SYN_PAGE * dim / 8) {
+        const int row = it / (dim / 8), c8 = it % (dim / 8);
+        *(uint4*)(Ks + row * KLD + 8 * c8) = kreg[r];
+      }
+      if (it < SYN_PAGE * vdim / 8) {
+        const int row = it / 8, c8 = it % 8;
+        uint2* dst = (uint2*)(Vs + row * VLD + 8 * c8);       // (a V row in LDS begins at a multiple of 8 bytes only)
+        dst[0] = make_uint2(vreg[r].x, vreg[r].y);
+        dst[1] = make_uint2(vreg[r].z, vreg[r].w);
       }
     }
   };
-  int page = page_table[(size_t)seq * table_stride + block_of(0)];
-  load_k(page);
+  fetch(0);
   for (int idx = 0; idx < n_blocks; ++idx) {
     const int kb = block_of(idx);
-    const bf16* vpage = v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
-    bf16x8 vf[2][AWP_TILES];
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
-#pragma unroll
-      for (int j = 0; j < AWP_TILES; ++j)
-        if (j < vt) {
-          // k index 8 g + e stands for key 32 pr + 4 g + e, 8 g + 4 + e for key 32 pr + 16 + 4 g + e (see below)
-          const bf16* vrow = vpage + (size_t)(16 * j + i) * SYN_PAGE + 32 * pr + 4 * g;
-          vf[pr][j] = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
-        }
+    __syncthreads();          // every wave has left the page before
+    stage();
+    __syncthreads();
+    if (idx + 1 < n_blocks) fetch(idx + 1);
+    const int page_lo = kb * SYN_PAGE, page_hi = page_lo + SYN_PAGE - 1;
+    if (!wave_on || page_lo > kmax_wave || (page_hi < lo_wave && page_lo >= terms.keep_first)) continue;   // none of it is seen
     f32x4 s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* krow = Ks + (16 * t + i) * KLD;
       if constexpr (X32) {
 #pragma unroll
         for (int c = 0; c < AWP_TILES / 2; ++c)
-          if (c < dim / 32) s[t] = awp_mfma32(kf8[t][c], qf8[c], s[t]);
+          if (c < dim / 32) s[t] = awp_mfma32(*(const bf16x8*)(krow + 32 * c + 8 * g), qf8[c], s[t]);
       } else {
 #pragma unroll
         for (int c = 0; c < AWP_TILES; ++c)
-          if (c < dim / 16) s[t] = awp_mfma16(kf4[t][c], qf4[c], s[t]);
+          if (c < dim / 16) s[t] = awp_mfma16(*(const bf16x4*)(krow + 16 * c + 4 * g), qf4[c], s[t]);
       }
-    }
-    if (idx + 1 < n_blocks) {
-      page = page_table[(size_t)seq * table_stride + block_of(idx + 1)];
-      load_k(page);
     }
     // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i)
     float mx = -INFINITY;
@@ -456,9 +467,11 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
 #pragma unroll
       for (int j = 0; j < AWP_TILES; ++j) {
         if (j < vt) {
+          const bf16* vrow = Vs + (16 * j + i) * VLD + 32 * pr + 4 * g;
+          const bf16x8 a = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
           if (pr == 0) O[j] *= alpha;
-          O[j] = awp_mfma32(vf[pr][j], b_hi, O[j]);
-          O[j] = awp_mfma32(vf[pr][j], b_lo, O[j]);
+          O[j] = awp_mfma32(a, b_hi, O[j]);
+          O[j] = awp_mfma32(a, b_lo, O[j]);
         }
       }
     }

@@ -749,10 +749,12 @@ def streams_read_norm(X, in_w, out, dyt=None, rows=None, delta=None):
           _is_f32(out), _stream())
 
 
-def streams_update(X, mix, out_w, terms):
+def streams_update(X, mix, out_w, terms, read=None):
     """X[n, t] = sum_s mix[s, t] X[n, s] + out_w[t] y[n] in place, all streams from the old ones;
     y = sum over `terms` of scale * (sum of the term's partial sums + bias).  terms: one or two (tensor [N, W] or
-    [P, N, W] float, scale, bias [W] float or None)."""
+    [P, N, W] float, scale, bias [W] float or None).
+    read = (in_w [S] float, dyt or None, out [N, W] bf16 or float): what the next sublayer reads leaves in the same
+    pass, out[n] = norm(sum_t in_w[t] X'[n, t]) with dyt as in streams_read_norm."""
     N, S, W = _streams(X, "streams_update.X")
     _need(mix, "streams_update.mix", _F32, (S, S))
     _need(out_w, "streams_update.out_w", _F32, (S,))
@@ -767,7 +769,20 @@ def streams_update(X, mix, out_w, terms):
             if bias is not None:
                 _need(bias, "streams_update.bias", _F32, (W,))
         args += [_ptr(y), parts, ctypes.c_float(scale), _ptr(bias)]
-    _call(load_library("core"), "syn_streams_update", _ptr(X), N, S, W, _ptr(mix), _ptr(out_w), *args, _stream())
+    nxt = [_ptr(None), ROWNORM_NONE, _ptr(None), _ptr(None), _ptr(None), _ptr(None), 0]
+    if read is not None:
+        in_w, dyt, out = read
+        _need(in_w, "streams_update.read.in_w", _F32, (S,))
+        _need(out, "streams_update.read.out", (_BF16, _F32), (N, W))
+        alpha = gain = shift = None
+        if dyt is not None:
+            alpha, gain, shift = dyt
+            _need(alpha, "streams_update.read.alpha", _F32)
+            _need(gain, "streams_update.read.gain", _F32, (W,))
+            _need(shift, "streams_update.read.shift", _F32, (W,))
+        nxt = [_ptr(in_w), ROWNORM_NONE if dyt is None else ROWNORM_DYT, _ptr(alpha), _ptr(gain), _ptr(shift), _ptr(out),
+               _is_f32(out)]
+    _call(load_library("core"), "syn_streams_update", _ptr(X), N, S, W, _ptr(mix), _ptr(out_w), *args, *nxt, _stream())
 
 
 def streams_start(x, X):

@@ -6,7 +6,7 @@ from .memory import MatrixMemory
 from .feedforward import FeedForward, GatedMlp
 from .block import Block, PreNormBlock, HyperConnectionBlock
 from .linear import (Matrix, linear, linear_for_sum, deferred_product, DeferredProduct, ScaledRows, WeightedDeltas,
-                     as_rows, as_delta)
+                     StreamsWrite, as_rows, as_delta)
 
 __all__ = ["Part", "KvNeed", "StateNeed", "flat_needs", "RmsNorm", "DynamicTanh", "Position", "NoPosition",
            "RotaryHalfSplit", "LogDistanceBias", "Mixer", "GqaAttention", "GatedWindowAttention", "ParallelMixers",

@@ -71,9 +71,10 @@ class HyperConnectionBlock(Block):
         u = sum_s in_q[s] X[s];   y = sublayer(norm_q(u));   X'[t] = sum_s mix_q[s, t] X[s] + out_q[t] y
 
     with all streams written at once from the old ones.  Tensors: prefix + "hc<q>.in" [S], ".out" [S], ".mix" [S, S]
-    (from, to).  Nothing is left pending: the block's last sum is made inside it.
+    (from, to).  A sublayer's result is written into the streams by the pass that gathers the next sublayer's input
+    (parts.linear.StreamsWrite): the block's last one leaves as `pending`, for the next block or the final norm.
     """
-    takes_deferred_product = False
+    takes_deferred_product = True       # `pending` may be the StreamsWrite that the block before left
 
     def __init__(self, prefix: str, streams: int, norm1, mixer, norm2=None, feed_forward=None,
                  names=("hc1.", "hc2.")):
@@ -115,30 +116,30 @@ class HyperConnectionBlock(Block):
         for p in self._parts():
             p.check(dtype)
 
-    def _read(self, norm, resid, in_w, dtype):
-        if hasattr(norm, "read"):
-            return norm.read(resid, in_w, dtype)
+    def _read(self, norm, resid, in_w, dtype, pending=None):
+        """The sublayer's input: the norm of the streams' weighted sum, after `pending` (a StreamsWrite) has been
+        written; one pass where the norm can be applied on the way."""
         import torch
         from ..kernels import ops
+        if pending is not None and hasattr(norm, "dyt_tensors"):
+            return pending.write_and_read(in_w, norm.dyt_tensors(), dtype)
+        if pending is not None:
+            pending.run()
+        if hasattr(norm, "read"):
+            return norm.read(resid, in_w, dtype)
         u = torch.empty((resid.shape[0], resid.shape[2]), dtype=torch.float32, device=resid.device)
         ops.streams_read_norm(resid, in_w, u)
         return norm.add_apply(u, None, dtype)
 
-    @staticmethod
-    def _write(resid, hc, y):
-        from ..kernels import ops
-        from .linear import WeightedDeltas
-        terms = y.terms if isinstance(y, WeightedDeltas) else [(as_delta(y), 1.0, None)]
-        ops.streams_update(resid, hc[2], hc[1], terms)
-
     def forward(self, resid, pending, ctx, cache, owner=True):
-        if pending is not None:
-            raise ValueError("a block over residual streams takes no pending delta")
+        from .linear import StreamsWrite
+        if pending is not None and not isinstance(pending, StreamsWrite):
+            raise ValueError("a block over residual streams takes no pending delta but another such block's")
         if resid.dim() != 3 or resid.shape[1] != self.streams:
             raise ValueError(f"the residual has shape {list(resid.shape)}; this block reads {self.streams} streams")
-        h = self._read(self.norm1, resid, self.hc[0][0], ctx.act_dtype)
-        self._write(resid, self.hc[0], self.mixer.forward(h, ctx, cache, owner))
+        h = self._read(self.norm1, resid, self.hc[0][0], ctx.act_dtype, pending)
+        pending = StreamsWrite(resid, self.hc[0][2], self.hc[0][1], self.mixer.forward(h, ctx, cache, owner))
         if self.feed_forward is not None:
-            h2 = self._read(self.norm2, resid, self.hc[1][0], ctx.act_dtype)
-            self._write(resid, self.hc[1], self.feed_forward.forward(h2, ctx))
-        return None
+            h2 = self._read(self.norm2, resid, self.hc[1][0], ctx.act_dtype, pending)
+            pending = StreamsWrite(resid, self.hc[1][2], self.hc[1][1], self.feed_forward.forward(h2, ctx))
+        return pending

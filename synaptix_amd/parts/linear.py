@@ -102,9 +102,30 @@ class WeightedDeltas:
         return zero
 
 
+class StreamsWrite:
+    """A sublayer's result on its way into a residual that runs in streams, not yet written:
+    X'[t] = sum_s mix[s, t] X[s] + out_w[t] y.  Whoever reads the streams next either takes it in, updating the
+    streams and gathering its own input in one pass (`write_and_read`), or asks for `run()`, which writes the
+    streams and leaves nothing to add (None)."""
+
+    def __init__(self, resid, mix, out_w, y):
+        self.resid, self.mix, self.out_w = resid, mix, out_w
+        self.terms = y.terms if isinstance(y, WeightedDeltas) else [(as_delta(y), 1.0, None)]
+
+    def run(self):
+        ops.streams_update(self.resid, self.mix, self.out_w, self.terms)
+        return None
+
+    def write_and_read(self, in_w, dyt, out_dtype):
+        """The streams written, and norm(sum_t in_w[t] X'[t]) of every row (dyt: a dynamic tanh's tensors or None)."""
+        out = torch.empty((self.resid.shape[0], self.resid.shape[-1]), dtype=out_dtype, device=self.resid.device)
+        ops.streams_update(self.resid, self.mix, self.out_w, self.terms, read=(in_w, dyt, out))
+        return out
+
+
 def as_delta(d):
     """The delta of the residual rows as a tensor (or None), whatever form it arrives in."""
-    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas)) else d
+    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas, StreamsWrite)) else d
 
 
 def deferred_product(x, w):

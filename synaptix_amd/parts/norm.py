@@ -85,6 +85,10 @@ class DynamicTanh(Part):
         self.alpha = get(self.alpha_name).float().reshape(1).contiguous()
         self.shift = get(self.shift_name).float().contiguous()
 
+    def dyt_tensors(self):
+        """(alpha, gain, shift): what the kernels that apply this norm on their way take."""
+        return self.alpha, self.gain, self.shift
+
     def read(self, resid, in_weights, out_dtype, rows=None, delta=None):
         """The norm of sum_s in_weights[s] * resid[:, s] (in_weights None: of the sum of the streams)."""
         n = resid.shape[0] if rows is None else rows.shape[0]

@@ -56,6 +56,14 @@ def test_streams_read_write_and_dynamic_tanh(S):
     ops.streams_update(X, dev(mix), dev(w_out), [(dev(ya), 0.8, dev(bias)), (dev(yb), -0.5, None)])
     want = P.streams_write(xs, mix, w_out, 0.8 * (ya.sum(0) + bias) - 0.5 * yb)
     assert float((X.cpu().double().permute(1, 0, 2) - want).abs().max()) < 5e-5
+    # the same update with the next sublayer's read leaving in the same pass
+    X2 = dev(xs.permute(1, 0, 2))
+    nxt = torch.empty((T, W), dtype=torch.float32, device=DEV)
+    w_next = torch.randn(S, generator=g, dtype=P.F64)
+    ops.streams_update(X2, dev(mix), dev(w_out), [(dev(ya), 0.8, dev(bias)), (dev(yb), -0.5, None)],
+                       read=(dev(w_next), (dev(alpha.reshape(1)), dev(gain), dev(shift)), nxt))
+    assert torch.equal(X2, X)
+    assert float((nxt.cpu().double() - P.dynamic_tanh(P.streams_read(want, w_next), alpha, gain, shift)).abs().max()) < 5e-5
     x0 = dev(xs[0])
     ops.streams_start(x0, X)
     assert torch.equal(X, x0.unsqueeze(1).expand(T, S, W))
