@@ -142,6 +142,7 @@ struct ChunkWork {     // scratch of one call; `chunks` is the most chunks the s
   float* S0;           // [chunks][H][dim][vdim]  the state before the chunk
   float* n0;           // [chunks][H][dim]
   float* m0;           // [chunks][H]
+  float* m_end;        // [sequences][H]  m behind a sequence's last chunk
 };
 
 // which sequence and which tokens chunk `c` of the step holds; false: there is no such chunk
@@ -252,72 +253,51 @@ mm_chunk_local_kernel(const float* __restrict__ proj, int width, const float* __
   }
 }
 
-// One workgroup for each (sequence, head, 64 columns): elementwise over the chunks of the sequence, in order.
-template <int DPT>
-__global__ void __launch_bounds__(MM_DG * SYN_WAVE)
+// Elementwise over the chunks of a sequence, in order: a thread carries one element of S (or of n) from chunk to
+// chunk, so that a (sequence, head) is spread over as many workgroups as its state has elements / 256.  m after the
+// last chunk goes to work.m_end (other workgroups still read the old m from the state): the out kernel stores it.
+__global__ void __launch_bounds__(256)
 mm_chunk_carry_kernel(float* __restrict__ state, int spare_row, const int* __restrict__ seq_start,
                       const int* __restrict__ seq_slot, ChunkWork work, int H, int dim, int vdim) {
-  const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
-  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
-  const int v = vt * MM_VT + lane;
-  const bool v_ok = v < vdim;
+  const int b = blockIdx.x, h = blockIdx.y;
+  const long SV = (long)dim * vdim, total = SV + dim;
+  const long e = (long)blockIdx.z * 256 + threadIdx.x;
   const int n_new = seq_start[b + 1] - seq_start[b];
   if (n_new <= 0) return;
   int c = 0;                      // the step's chunks before this sequence's
   for (int x = 0; x < b; ++x) c += (seq_start[x + 1] - seq_start[x] + MMC_L - 1) / MMC_L;
   const int n_chunks = (n_new + MMC_L - 1) / MMC_L;
   const int slot = seq_slot[b];
-  const size_t per_head = (size_t)dim * vdim + dim + 1;
-  float* st = state + ((size_t)(slot < 0 ? spare_row : slot) * H + h) * per_head;
-  float S[DPT], U[DPT];
+  float* st = state + ((size_t)(slot < 0 ? spare_row : slot) * H + h) * (total + 1);
+  const bool on = e < total, is_s = e < SV, first = blockIdx.z == 0 && threadIdx.x == 0;
+  float x = on ? st[e] : 0.f;
+  float m = st[total];
+  constexpr int AHEAD = 4;         // chunks whose sums are asked for together
+  for (int k0 = 0; k0 < n_chunks; k0 += AHEAD) {
+    float u[AHEAD], bL[AHEAD], PL[AHEAD];
 #pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = wave + MM_DG * j;
-    S[j] = (d < dim && v_ok) ? st[(size_t)d * vdim + v] : 0.f;
-  }
-  const int dn = wave + MM_DG * lane;
-  float n = dn < dim ? st[(size_t)dim * vdim + dn] : 0.f;
-  float m = st[(size_t)dim * vdim + dim];
-  auto load_u = [&](int cc) {
-    const float* Uc = work.U + ((size_t)cc * H + h) * dim * vdim;
-#pragma unroll
-    for (int j = 0; j < DPT; ++j) {
-      const int d = wave + MM_DG * j;
-      U[j] = (d < dim && v_ok) ? Uc[(size_t)d * vdim + v] : 0.f;
+    for (int a = 0; a < AHEAD; ++a) {
+      const size_t ch = (size_t)(c + min(k0 + a, n_chunks - 1)) * H + h;
+      u[a] = !on ? 0.f : (is_s ? work.U[ch * SV + e] : work.un[ch * dim + (e - SV)]);
+      bL[a] = work.stat[ch * 2], PL[a] = work.stat[ch * 2 + 1];
     }
-  };
-  load_u(c);
-  for (int k = 0; k < n_chunks; ++k, ++c) {
-    const size_t ch = (size_t)c * H + h;
-    const float bL = work.stat[ch * 2], PL = work.stat[ch * 2 + 1];
-    const float un = dn < dim ? work.un[ch * dim + dn] : 0.f;
-    float* S0 = work.S0 + ch * dim * vdim;
 #pragma unroll
-    for (int j = 0; j < DPT; ++j) {
-      const int d = wave + MM_DG * j;
-      if (d < dim && v_ok) S0[(size_t)d * vdim + v] = S[j];
+    for (int a = 0; a < AHEAD; ++a) {
+      if (k0 + a < n_chunks) {
+        const size_t ch = (size_t)(c + k0 + a) * H + h;
+        if (on) {
+          if (is_s) work.S0[ch * SV + e] = x;
+          else work.n0[ch * dim + (e - SV)] = x;
+        }
+        if (first) work.m0[ch] = m;
+        const float M = fmaxf(m, PL[a]);
+        x = expf(m - M) * x + expf(PL[a] - M) * u[a];
+        m = bL[a] + M;
+      }
     }
-    if (vt == 0) {
-      if (dn < dim) work.n0[ch * dim + dn] = n;
-      if (threadIdx.x == 0) work.m0[ch] = m;
-    }
-    const float M = fmaxf(m, PL);
-    const float keep = expf(m - M), take = expf(PL - M);
-#pragma unroll
-    for (int j = 0; j < DPT; ++j) S[j] = keep * S[j] + take * U[j];
-    n = keep * n + take * un;
-    m = bL + M;
-    if (k + 1 < n_chunks) load_u(c + 1);
   }
-#pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = wave + MM_DG * j;
-    if (d < dim && v_ok) st[(size_t)d * vdim + v] = S[j];
-  }
-  if (vt == 0) {
-    if (dn < dim) st[(size_t)dim * vdim + dn] = n;
-    if (threadIdx.x == 0) st[(size_t)dim * vdim + dim] = m;
-  }
+  if (on) st[e] = x;
+  if (first) work.m_end[(size_t)b * H + h] = m;
 }
 
 __host__ __device__ inline size_t mmc_out_lds_floats(int dim) {
@@ -327,7 +307,8 @@ __host__ __device__ inline size_t mmc_out_lds_floats(int dim) {
 __global__ void __launch_bounds__(MM_DG * SYN_WAVE)
 mm_chunk_out_kernel(const float* __restrict__ proj, int width, const float* __restrict__ i_bias,
                     const float* __restrict__ f_bias, float cap, float q_scale, const int* __restrict__ seq_start,
-                    int n_seqs, ChunkWork work, float* __restrict__ out, int H, int dim, int vdim) {
+                    int n_seqs, ChunkWork work, float* __restrict__ out, int H, int dim, int vdim,
+                    float* __restrict__ state, int spare_row, const int* __restrict__ seq_slot) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int L = MMC_L;
   const int DP = dim + 1;
@@ -349,6 +330,12 @@ mm_chunk_out_kernel(const float* __restrict__ proj, int width, const float* __re
   const int v = vt * MM_VT + lane;
   const bool v_ok = v < vdim;
   const size_t ch = (size_t)c * H + h;
+  if (first == seq_start[seq] && vt == 0 && tid == 0) {
+    // the sequence's m behind this step, which the carry left aside
+    const int slot = seq_slot[seq];
+    state[((size_t)(slot < 0 ? spare_row : slot) * H + h) * ((size_t)dim * vdim + dim + 1) + (size_t)dim * vdim + dim] =
+        work.m_end[(size_t)seq * H + h];
+  }
   const int q_col = h * dim, k_col = H * dim + h * dim, v_col = 2 * H * dim + h * vdim;
   const int i_col = 2 * H * dim + 2 * H * vdim + h, f_col = i_col + H;
   for (int idx = tid; idx < L * dim; idx += blockDim.x) {
@@ -451,7 +438,7 @@ static hipError_t raise_chunk_out_lds() {
 // floats of scratch memory that a chunked call over n_tokens tokens in n_seqs sequences needs
 SYN_EXPORT long syn_matrix_memory_chunk_scratch(int n_tokens, int n_seqs, int H, int dim, int vdim) {
   const long chunks = (n_tokens + MMC_L - 1) / MMC_L + n_seqs;
-  return chunks * H * (2L * dim * vdim + 2L * dim + 3);
+  return chunks * H * (2L * dim * vdim + 2L * dim + 3) + (long)n_seqs * H;
 }
 
 // out [N][H * vdim] float: o_t of every token, before the heads' norm
@@ -478,6 +465,8 @@ SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float*
     w.n0 = w.un + chunks * H * dim;
     w.stat = w.n0 + chunks * H * dim;
     w.m0 = w.stat + chunks * H * 2;
+    w.m_end = w.m0 + chunks * H;
+    const dim3 carry_grid(n_seqs, H, (unsigned)(((long)dim * vdim + dim + 255) / 256));
     const dim3 per_chunk((unsigned)chunks, H, (vdim + MM_VT - 1) / MM_VT);
     const size_t local_lds = ((size_t)MMC_L * (dim + 1) + MMC_L * MM_VT + MMC_L) * sizeof(float);
     const size_t out_lds = mmc_out_lds_floats(dim) * sizeof(float);
@@ -487,16 +476,16 @@ SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float*
   do {                                                                                                                   \
     mm_chunk_local_kernel<D><<<per_chunk, MM_DG * SYN_WAVE, local_lds, stream>>>(proj, width, i_bias, f_bias, cap,        \
                                                                                  seq_start, n_seqs, w, H, dim, vdim);     \
-    mm_chunk_carry_kernel<D><<<grid, MM_DG * SYN_WAVE, 0, stream>>>(state, state_rows - 1, seq_start, seq_slot, w, H,    \
-                                                                    dim, vdim);                                          \
   } while (0)
     if (dpt <= 8) SYN_MMC(8);
     else if (dpt <= 16) SYN_MMC(16);
     else if (dpt <= 32) SYN_MMC(32);
     else SYN_MMC(64);
 #undef SYN_MMC
+    mm_chunk_carry_kernel<<<carry_grid, 256, 0, stream>>>(state, state_rows - 1, seq_start, seq_slot, w, H, dim, vdim);
     mm_chunk_out_kernel<<<per_chunk, MM_DG * SYN_WAVE, out_lds, stream>>>(proj, width, i_bias, f_bias, cap, q_scale,
-                                                                          seq_start, n_seqs, w, out, H, dim, vdim);
+                                                                          seq_start, n_seqs, w, out, H, dim, vdim, state,
+                                                                          state_rows - 1, seq_slot);
     SYN_LAUNCH_CHECK("matrix_memory_scan (chunks)");
     return 0;
   }
