@@ -450,3 +450,51 @@ def test_short_prompt_steps_replayed_from_a_graph():
         at += n
         assert_logits_close(got, want[at - 1:at], "bfloat16", f"prompt portion ending at {at} through a graph", sharp=True)
     assert any(k[0] == "prompt" for k in eng._runners), "no prompt step was replayed from a graph"
+
+
+def test_command_line_and_trace_replay_as_a_user_starts_them(tmp_path):
+    """`random` writes a model folder from a configuration file, `run` generates from it, and bin/trace_run replays
+    steps over it (prompts of unequal lengths together, then single tokens, a request that ends early, its slot used
+    again by a later request) in both types; the logits against the plain model, the generated tokens against its
+    greedy choice."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from helpers import ROOT, batched_trace
+    from plain_bizipel import PlainBizipel
+
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(CONFIGS["P"]))
+    folder = str(tmp_path / "model")
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    subprocess.run([sys.executable, "-m", "synaptix_amd", "random", str(cfg_file), folder, "--seed", "3"], check=True,
+                   env=env, cwd=ROOT, timeout=300)
+    plain = PlainBizipel.from_folder(folder)
+    prompt = tokens_for("P", 9, 1)
+    run = subprocess.run([sys.executable, "-m", "synaptix_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)),
+                          "--max-tokens", "6", "--temperature", "0", "--compute-dtype", "f32"], check=True, env=env,
+                         cwd=ROOT, timeout=300, capture_output=True, text=True)
+    out = [int(t) for t in run.stdout.split()]
+    assert len(out) == 6
+    logits = plain.forward(prompt + out)
+    for i, tok in enumerate(out):
+        row = logits[len(prompt) - 1 + i]
+        assert tok == int(row.argmax()) or float(row.max() - row[tok]) < 1e-4
+
+    reqs = {"a": tokens_for("P", 75, 2), "b": tokens_for("P", 8, 3), "c": tokens_for("P", 130, 4), "d": tokens_for("P", 40, 5)}
+    steps, where = batched_trace(reqs, [["a", "b", "c"], ["d", "b"]], decode=5)
+    for dtype in DTYPES:
+        out_dir = str(tmp_path / dtype)
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                               "--out", out_dir, "--max-tokens", "640"], input="".join(json.dumps(s) + "\n" for s in steps),
+                              capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]
+        got = {s["step"]: np.fromfile(os.path.join(out_dir, f"{s['step']}.f32"), dtype="<f4").reshape(-1, CONFIGS["P"]["vocab"])
+               for s in steps}
+        for rid, toks in reqs.items():
+            want = plain.forward(toks)
+            rows = np.stack([got[where[(rid, p)][0]][where[(rid, p)][1]] for p in range(len(toks))])
+            assert_logits_close(rows, want, dtype, f"trace_run {dtype} request {rid}", sharp=False)
