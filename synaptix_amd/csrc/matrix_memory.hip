@@ -18,8 +18,9 @@
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-// One workgroup for each (sequence of the step, head, tile of 64 columns); it walks the sequence's new tokens in order
-// with its part of S in registers.  Tile 0 also keeps n and m for the state (every tile computes them).
+// One workgroup for each (sequence of the step, head); it walks the sequence's new tokens in order with 64 columns of S
+// in registers, one tile of 64 columns after another.  n and m are read once, carried anew from there in every pass over
+// a tile (the same values each time), and stored after the last: no other workgroup reads or writes this head's state.
 template <int DPT>   // rows of S a thread keeps: dim <= 4 * DPT
 __global__ void __launch_bounds__(MM_DG * SYN_WAVE)
 matrix_memory_scan_kernel(const float* __restrict__ proj, int width, const float* __restrict__ i_bias,
@@ -31,10 +32,8 @@ matrix_memory_scan_kernel(const float* __restrict__ proj, int width, const float
   __shared__ float gs[MM_TC][2];
   __shared__ float red[2][MM_DG][MM_VT];
   __shared__ float red_n[2][MM_DG];
-  const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
+  const int b = blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
-  const int v = vt * MM_VT + lane;
-  const bool v_ok = v < vdim;
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
   if (t0 >= t1) return;     // a sequence without tokens in this step (the spare ones of a padded step): nothing moves
   const int slot = seq_slot[b];
@@ -43,81 +42,84 @@ matrix_memory_scan_kernel(const float* __restrict__ proj, int width, const float
   const int q_col = h * dim, k_col = H * dim + h * dim, v_col = 2 * H * dim + h * vdim;
   const int i_col = 2 * H * dim + 2 * H * vdim + h, f_col = i_col + H;
   const float bi = i_bias ? i_bias[h] : 0.f, bf = f_bias ? f_bias[h] : 0.f;
-
-  float S[DPT];
-#pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = wave + MM_DG * j;
-    S[j] = (d < dim && v_ok) ? st[(size_t)d * vdim + v] : 0.f;
-  }
   const int dn = wave + MM_DG * lane;          // the entry of n this thread keeps
-  float n = dn < dim ? st[(size_t)dim * vdim + dn] : 0.f;
-  float m = st[(size_t)dim * vdim + dim];
+  const float n_before = dn < dim ? st[(size_t)dim * vdim + dn] : 0.f;
+  const float m_before = st[(size_t)dim * vdim + dim];
+  float n = n_before, m = m_before;
 
-  for (int c0 = t0; c0 < t1; c0 += MM_TC) {
-    const int nc = min(MM_TC, t1 - c0);
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < nc * dim; idx += blockDim.x) {
-      const int t = idx / dim, d = idx % dim;
-      const float* row = proj + (size_t)(c0 + t) * width;
-      qs[t][d] = row[q_col + d] * q_scale;
-      ks[t][d] = row[k_col + d];
+  for (int vt = 0; vt * MM_VT < vdim; ++vt) {
+    const int v = vt * MM_VT + lane;
+    const bool v_ok = v < vdim;
+    n = n_before, m = m_before;
+    float S[DPT];
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) {
+      const int d = wave + MM_DG * j;
+      S[j] = (d < dim && v_ok) ? st[(size_t)d * vdim + v] : 0.f;
     }
-    if (threadIdx.x < nc * 2) {
-      const int t = threadIdx.x / 2, which = threadIdx.x % 2;
-      const float raw = proj[(size_t)(c0 + t) * width + (which ? f_col : i_col)] + (which ? bf : bi);
-      const float capped = cap > 0.f ? cap * tanhf(raw / cap) : raw;
-      gs[t][which] = which ? log_sigmoid(capped) : capped;
-    }
-    float vv[MM_TC];
+    for (int c0 = t0; c0 < t1; c0 += MM_TC) {
+      const int nc = min(MM_TC, t1 - c0);
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < nc * dim; idx += blockDim.x) {
+        const int t = idx / dim, d = idx % dim;
+        const float* row = proj + (size_t)(c0 + t) * width;
+        qs[t][d] = row[q_col + d] * q_scale;
+        ks[t][d] = row[k_col + d];
+      }
+      if (threadIdx.x < nc * 2) {
+        const int t = threadIdx.x / 2, which = threadIdx.x % 2;
+        const float raw = proj[(size_t)(c0 + t) * width + (which ? f_col : i_col)] + (which ? bf : bi);
+        const float capped = cap > 0.f ? cap * tanhf(raw / cap) : raw;
+        gs[t][which] = which ? log_sigmoid(capped) : capped;
+      }
+      float vv[MM_TC];
 #pragma unroll
-    for (int t = 0; t < MM_TC; ++t) vv[t] = (t < nc && v_ok) ? proj[(size_t)(c0 + t) * width + v_col + v] : 0.f;
-    __syncthreads();
+      for (int t = 0; t < MM_TC; ++t) vv[t] = (t < nc && v_ok) ? proj[(size_t)(c0 + t) * width + v_col + v] : 0.f;
+      __syncthreads();
 #pragma unroll
-    for (int t = 0; t < MM_TC; ++t) {
-      if (t < nc) {
-        const float ig = gs[t][0], fg = gs[t][1];
-        const float m_new = fmaxf(fg + m, ig);
-        const float a = expf(fg + m - m_new), bb = expf(ig - m_new);
-        m = m_new;
-        float num = 0.f;
+      for (int t = 0; t < MM_TC; ++t) {
+        if (t < nc) {
+          const float ig = gs[t][0], fg = gs[t][1];
+          const float m_new = fmaxf(fg + m, ig);
+          const float a = expf(fg + m - m_new), bb = expf(ig - m_new);
+          m = m_new;
+          float num = 0.f;
 #pragma unroll
-        for (int j = 0; j < DPT; ++j) {
-          const int d = wave + MM_DG * j;
-          if (d < dim) {
-            S[j] = a * S[j] + (bb * ks[t][d]) * vv[t];
-            num = fmaf(S[j], qs[t][d], num);
+          for (int j = 0; j < DPT; ++j) {
+            const int d = wave + MM_DG * j;
+            if (d < dim) {
+              S[j] = a * S[j] + (bb * ks[t][d]) * vv[t];
+              num = fmaf(S[j], qs[t][d], num);
+            }
           }
-        }
-        float nq = 0.f;
-        if (dn < dim) {
-          n = a * n + bb * ks[t][dn];
-          nq = n * qs[t][dn];
-        }
-        nq = wave_sum(nq);
-        const int buf = t & 1;
-        red[buf][wave][lane] = num;
-        if (lane == 0) red_n[buf][wave] = nq;
-        __syncthreads();
-        if (wave == 0 && v_ok) {
-          float total = 0.f, nqt = 0.f;
+          float nq = 0.f;
+          if (dn < dim) {
+            n = a * n + bb * ks[t][dn];
+            nq = n * qs[t][dn];
+          }
+          nq = wave_sum(nq);
+          const int buf = t & 1;
+          red[buf][wave][lane] = num;
+          if (lane == 0) red_n[buf][wave] = nq;
+          __syncthreads();
+          if (wave == 0 && v_ok) {
+            float total = 0.f, nqt = 0.f;
 #pragma unroll
-          for (int w = 0; w < MM_DG; ++w) total += red[buf][w][lane], nqt += red_n[buf][w];
-          const float den = fmaxf(fabsf(nqt), expf(-m)) + 1e-6f;
-          out[(size_t)(c0 + t) * H * vdim + (size_t)h * vdim + v] = total / den;
+            for (int w = 0; w < MM_DG; ++w) total += red[buf][w][lane], nqt += red_n[buf][w];
+            const float den = fmaxf(fabsf(nqt), expf(-m)) + 1e-6f;
+            out[(size_t)(c0 + t) * H * vdim + (size_t)h * vdim + v] = total / den;
+          }
         }
       }
     }
-  }
 #pragma unroll
-  for (int j = 0; j < DPT; ++j) {
-    const int d = wave + MM_DG * j;
-    if (d < dim && v_ok) st[(size_t)d * vdim + v] = S[j];
+    for (int j = 0; j < DPT; ++j) {
+      const int d = wave + MM_DG * j;
+      if (d < dim && v_ok) st[(size_t)d * vdim + v] = S[j];
+    }
   }
-  if (vt == 0) {
-    if (dn < dim) st[(size_t)dim * vdim + dn] = n;
-    if (threadIdx.x == 0) st[(size_t)dim * vdim + dim] = m;
-  }
+  if (dn < dim) st[(size_t)dim * vdim + dn] = n;
+  if (threadIdx.x == 0) st[(size_t)dim * vdim + dim] = m;
 }
 
 // The same cell for prompts, in chunks of MMC_L tokens that are worked on side by side.  Inside a chunk, with b_t the
@@ -489,9 +491,11 @@ SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float*
     SYN_LAUNCH_CHECK("matrix_memory_scan (chunks)");
     return 0;
   }
-#define SYN_MM(D)                                                                                                   \
-  matrix_memory_scan_kernel<D><<<grid, MM_DG * SYN_WAVE, 0, stream>>>(proj, width, i_bias, f_bias, cap, q_scale, state, \
-                                                                      state_rows - 1, seq_start, seq_slot, out, H, dim, vdim)
+  const dim3 per_head(n_seqs, H);
+#define SYN_MM(D)                                                                                                       \
+  matrix_memory_scan_kernel<D><<<per_head, MM_DG * SYN_WAVE, 0, stream>>>(proj, width, i_bias, f_bias, cap, q_scale, state, \
+                                                                          state_rows - 1, seq_start, seq_slot, out, H, dim, \
+                                                                          vdim)
   if (dpt <= 8) SYN_MM(8);
   else if (dpt <= 16) SYN_MM(16);
   else if (dpt <= 32) SYN_MM(32);

@@ -22,6 +22,7 @@ def test_configuration_round_trip_and_registry():
     cfg = BizipelConfig.from_dict(CONFIGS["P"])
     assert cfg.layers[0].left.window == 20 and cfg.layers[0].left.keep_first == 3 and cfg.layers[1].ff is None
     assert cfg.streams == 2 and BizipelConfig.from_dict(CONFIGS["Q"]).streams == 1
+    assert BizipelConfig.from_dict(CONFIGS["T"]).streams is None
     assert BizipelConfig.from_dict(config(10, 8, None, [layer(1, 1, 4, 4, 8, 0, 1, 4, 4, 8)])).streams is None
 
 

@@ -274,11 +274,12 @@ def test_matrix_memory_in_portions_and_slots(H, D, E, T, chunked):
 # ----------------------------------------------------------------------------- whole models
 
 def lengths(name):
-    return {"P": [1, 2, 21, 64, 65, 150], "Q": [3, 70, 71, 129, 140], "R": [5, 64, 128, 200]}[name]
+    return {"P": [1, 2, 21, 64, 65, 150], "Q": [3, 70, 71, 129, 140], "R": [5, 64, 128, 200], "S": [1, 12, 66, 90],
+            "T": [2, 31, 64, 100]}[name]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
 def test_whole_prompts(name, dtype):
     eng = engine(name, dtype)
     for i, n in enumerate(lengths(name)):
@@ -307,7 +308,7 @@ def test_portions_of_several_sizes(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,head,n", [("P", 30, 130), ("Q", 1, 160), ("R", 100, 140)])
+@pytest.mark.parametrize("name,head,n", [("P", 30, 130), ("Q", 1, 160), ("R", 100, 140), ("S", 3, 90), ("T", 40, 110)])
 def test_prompt_then_token_by_token(name, head, n, dtype):
     """Decoding long enough that every window passes over decoded tokens and over a page's border, that the kept first
     keys are the only old ones left, and that the state has been carried over a hundred steps."""
@@ -324,7 +325,7 @@ def test_prompt_then_token_by_token(name, head, n, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
 def test_unequal_batches_and_slots_used_again(name, dtype):
     """Requests of unequal lengths start together and are decoded together, the shorter ones ending earlier; then
     other requests take the slots and pages that came free (the cache has room for little more than one batch), in
