@@ -309,7 +309,7 @@ __device__ __forceinline__ bf16x8 awp_join(bf16x4 lo, bf16x4 hi) {
 #define AWP_VPAD 4      // the same for a V row (64 tokens)
 
 template <bool X32>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)      // (two waves a SIMD: the registers are bounded for that)
 window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                            const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                            const int* __restrict__ seq_past, int n_seqs, const float* __restrict__ gate, int gate_stride,
@@ -361,7 +361,9 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
   const int n_blocks = n_kept_blocks + (kmax / SYN_PAGE - first_window_block + 1);
   const float slope = terms.slopes ? terms.slopes[head] : 0.f;
   const float r1 = terms.r1 ? terms.r1[head] : 0.f, r2 = terms.r1 ? terms.r2[head] : 0.f;
-  float m = terms.sink_one ? 0.f : -INFINITY, l = terms.sink_one ? 1.f : 0.f;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = scale * LOG2E, slope2 = slope * LOG2E, cap2 = terms.softcap * LOG2E;
+  float m = terms.sink_one ? 0.f : -INFINITY, l = terms.sink_one ? 1.f : 0.f;     // (the sink's score 0 is 0 in any unit)
   f32x4 O[AWP_TILES];
 #pragma unroll
   for (int j = 0; j < AWP_TILES; ++j) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -370,6 +372,13 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
   // up to four of each), one page ahead of the page that is being multiplied, and from there into LDS.
   constexpr int PIECES = 16 * AWP_TILES * SYN_PAGE / 8 / 256;      // 4
   uint4 kreg[PIECES], vreg[PIECES];
+  int k_at[PIECES], v_at[PIECES];       // where this thread's pieces go in LDS (-1: the page has fewer pieces)
+#pragma unroll
+  for (int r = 0; r < PIECES; ++r) {
+    const int it = tid + 256 * r;
+    k_at[r] = it < SYN_PAGE * dim / 8 ? (it / (dim / 8)) * KLD + 8 * (it % (dim / 8)) : -1;
+    v_at[r] = it < SYN_PAGE * vdim / 8 ? (it / 8) * VLD + 8 * (it % 8) : -1;
+  }
   auto block_of = [&](int idx) { return idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks); };
   auto fetch = [&](int idx) {
     const int page = page_table[(size_t)seq * table_stride + block_of(idx)];
@@ -378,21 +387,16 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
       const int it = tid + 256 * r;
-      if (it < SYN_PAGE * dim / 8) kreg[r] = kp[it];
-      if (it < SYN_PAGE * vdim / 8) vreg[r] = vp[it];
+      if (k_at[r] >= 0) kreg[r] = kp[it];
+      if (v_at[r] >= 0) vreg[r] = vp[it];
     }
   };
   auto stage = [&]() {
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
-      const int it = tid + 256 * r;
-      if (it < SYN_PAGE * dim / 8) {
-        const int row = it / (dim / 8), c8 = it % (dim / 8);
-        *(uint4*)(Ks + row * KLD + 8 * c8) = kreg[r];
-      }
-      if (it < SYN_PAGE * vdim / 8) {
-        const int row = it / 8, c8 = it % 8;
-        uint2* dst = (uint2*)(Vs + row * VLD + 8 * c8);       // (a V row in LDS begins at a multiple of 8 bytes only)
+      if (k_at[r] >= 0) *(uint4*)(Ks + k_at[r]) = kreg[r];
+      if (v_at[r] >= 0) {
+        uint2* dst = (uint2*)(Vs + v_at[r]);       // (a V row in LDS begins at a multiple of 8 bytes only)
         dst[0] = make_uint2(vreg[r].x, vreg[r].y);
         dst[1] = make_uint2(vreg[r].z, vreg[r].w);
       }
@@ -422,20 +426,26 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
           if (c < dim / 16) s[t] = awp_mfma16(*(const bf16x4*)(krow + 16 * c + 4 * g), qf4[c], s[t]);
       }
     }
-    // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i)
+    // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i); a page that
+    // lies behind the wave's first query and inside its last query's window is seen whole by all of them: no mask
+    const bool whole = page_hi <= past + n0 && (W <= 0 || page_lo >= kmax_wave - W + 1);
+    const float dist0 = (float)(qpos - page_lo - 4 * g);
+    // scores in units of ln 2 from here on (scale, slope and cap carry log2 e; r1 ln(x) = r1 log2(x) ln 2): the
+    // exponentials below are bare exp2
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int key = kb * SYN_PAGE + 16 * t + 4 * g + e;
-        const bool valid = key <= qpos && (key >= lo_q || key < terms.keep_first);
-        float v = s[t][e] * scale;
-        if (terms.softcap > 0.f) v = terms.softcap * tanhf(v / terms.softcap);
-        const float dist = (float)(qpos - key);
-        v -= slope * dist;
-        if (terms.r1) v -= r1 * __logf(1.f + r2 * dist);
-        v = valid ? v : -INFINITY;
+        float v = s[t][e] * scale2;
+        if (terms.softcap > 0.f) v = cap2 * tanhf(s[t][e] * scale / terms.softcap);
+        const float dist = dist0 - (float)(16 * t + e);          // query position - key position
+        if (slope2 != 0.f) v -= slope2 * dist;
+        if (terms.r1) v -= r1 * __builtin_amdgcn_logf(fmaf(r2, dist, 1.f));
+        if (!whole) {
+          const int key = page_lo + 16 * t + 4 * g + e;
+          v = (key <= qpos && (key >= lo_q || key < terms.keep_first)) ? v : -INFINITY;
+        }
         s[t][e] = v;
         mx = fmaxf(mx, v);
       }
@@ -443,33 +453,39 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
     mx = fmaxf(mx, __shfl_xor(mx, 32, SYN_WAVE));
     const float m_new = fmaxf(m, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing seen yet: every weight below is zero
-    const float alpha = __expf(m - m_use);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
     float sum = 0.f;
-    bf16x4 hi[4], lw[4];
+    // a weight as two bf16 numbers: its upper 16 bits, and the upper 16 bits of what they leave (16 bits of mantissa
+    // together); two neighbours share a register
+    unsigned hi[4][2], lw[4][2];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float p = __expf(s[t][e] - m_use);      // exp(-inf) = 0 for what is hidden
-        sum += p;
-        const bf16 h = (bf16)p;
-        hi[t][e] = h;
-        lw[t][e] = (bf16)(p - (float)h);
+      for (int e = 0; e < 4; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(s[t][e] - m_use), p1 = __builtin_amdgcn_exp2f(s[t][e + 1] - m_use);
+        sum += p0 + p1;                                           // exp2(-inf) = 0 for what is hidden
+        const unsigned b0 = __float_as_uint(p0) & 0xffff0000u, b1 = __float_as_uint(p1) & 0xffff0000u;
+        hi[t][e / 2] = (b0 >> 16) | b1;
+        const unsigned r0 = __float_as_uint(p0 - __uint_as_float(b0)), r1b = __float_as_uint(p1 - __uint_as_float(b1));
+        lw[t][e / 2] = (r0 >> 16) | (r1b & 0xffff0000u);
       }
     sum += __shfl_xor(sum, 16, SYN_WAVE);
     sum += __shfl_xor(sum, 32, SYN_WAVE);
     l = l * alpha + sum;
     m = m_new;
+    const bool rescale = __any(alpha != 1.f);       // (the maximum moves in the first pages and then seldom)
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr) {
       // k index 8 g + e stands for key 32 pr + 4 g + e, 8 g + 4 + e for key 32 pr + 16 + 4 g + e: both operands agree
-      const bf16x8 b_hi = awp_join(hi[2 * pr], hi[2 * pr + 1]), b_lo = awp_join(lw[2 * pr], lw[2 * pr + 1]);
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+      const bf16x8 b_hi = __builtin_bit_cast(bf16x8, (u32x4){hi[2 * pr][0], hi[2 * pr][1], hi[2 * pr + 1][0], hi[2 * pr + 1][1]});
+      const bf16x8 b_lo = __builtin_bit_cast(bf16x8, (u32x4){lw[2 * pr][0], lw[2 * pr][1], lw[2 * pr + 1][0], lw[2 * pr + 1][1]});
 #pragma unroll
       for (int j = 0; j < AWP_TILES; ++j) {
         if (j < vt) {
           const bf16* vrow = Vs + (16 * j + i) * VLD + 32 * pr + 4 * g;
           const bf16x8 a = awp_join(*(const bf16x4*)vrow, *(const bf16x4*)(vrow + 16));
-          if (pr == 0) O[j] *= alpha;
+          if (pr == 0 && rescale) O[j] *= alpha;
           O[j] = awp_mfma32(a, b_hi, O[j]);
           O[j] = awp_mfma32(a, b_lo, O[j]);
         }
