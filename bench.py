@@ -22,7 +22,7 @@ own clock over its last `steps` decode steps, to stand beside `value`), the 4b w
 (decode_4b_unequal16, its fraction of the HBM roofline and its prompts' rate) and the 32b shape at
 8 sequences (decode_32b_b8), each with the sizes it ran at as a text.
 
---design bizipel: not the contract's run.  Prefill and decode throughput of the Bizipel design at a few layer sizes
+--design bizipel: another run than the default one.  Prefill and decode throughput of the Bizipel design at a few layer sizes
 beside the Qwen3 decoder at the same sizes (width, heads, head size, feed-forward, vocabulary, layers; random bf16
 weights), each with the time of every kernel entry point of one prompt step and one decode step; one JSON line.
 
@@ -284,7 +284,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--design", default=None, choices=["bizipel"],
-                    help="not the contract's run: this design beside the Qwen3 decoder at equal layer sizes")
+                    help="another run than the default one: this design beside the Qwen3 decoder at equal layer sizes")
     ap.add_argument("--sizes", default="small,mid,large", help="with --design: which of small, mid, large")
     ap.add_argument("--window", type=int, default=1024, help="with --design: the keys a query of the new design sees")
     args = ap.parse_args()
