@@ -41,13 +41,14 @@ def config(vocab, width, streams, layers, eps=1e-6):
 # T: no `streams` key at all: one plain residual with pre-norm layers.
 CONFIGS = {
     "S": config(101, 72, 3, [layer(2, 1, 20, 12, 10, 2, 1, 3, 5, 24), layer(3, 3, 12, 20, 1, 0, 2, 7, 9, 40, cap=20.0)]),
+    "U": config(77, 50, 2, [layer(1, 1, 6, 10, 3, 1, 1, 4, 6, 22)]),          # a width that is no multiple of 4
     "T": config(200, 64, None, [layer(2, 2, 16, 16, 30, 1, 1, 8, 8, 48), layer(4, 1, 8, 32, 200, 0, 2, 16, 24, 64)]),
     "P": config(300, 64, 2, [layer(4, 2, 16, 24, 20, 3, 2, 8, 16, 96), layer(2, 1, 32, 16, 70, 0, 1, 24, 40, None)]),
     "Q": config(257, 88, 1, [layer(3, 1, 24, 8, 64, 70, 1, 10, 72, 50, cap=3.0), layer(2, 2, 8, 40, 5, 1, 3, 6, 4, 120),
                              layer(1, 1, 40, 40, 33, 2, 2, 16, 16, 64, scales=(1.0, 1.0))], eps=1e-5),
     "R": config(512, 128, 4, [layer(4, 4, 32, 32, 4096, 0, 2, 32, 64, 256), layer(4, 4, 32, 32, 100, 8, 2, 32, 64, 256)]),
 }
-SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14, "T": 15}
+SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14, "T": 15, "U": 16}
 _tmp = None
 _folders, _plain, _logits = {}, {}, {}
 

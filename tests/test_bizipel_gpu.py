@@ -33,11 +33,12 @@ def dev(t, dtype=torch.float32):
 
 # ----------------------------------------------------------------------------- mechanisms alone
 
+@pytest.mark.parametrize("W", [72, 70])
 @pytest.mark.parametrize("S", [1, 2, 5])
-def test_streams_read_write_and_dynamic_tanh(S):
+def test_streams_read_write_and_dynamic_tanh(S, W):
     from synaptix_amd.kernels import ops
     g = torch.Generator().manual_seed(S)
-    T, W = 37, 72
+    T = 37
     xs = torch.randn(S, T, W, generator=g, dtype=P.F64) * 3
     w_in, w_out = torch.randn(S, generator=g, dtype=P.F64), torch.randn(S, generator=g, dtype=P.F64)
     mix = torch.randn(S, S, generator=g, dtype=P.F64)
@@ -275,11 +276,11 @@ def test_matrix_memory_in_portions_and_slots(H, D, E, T, chunked):
 
 def lengths(name):
     return {"P": [1, 2, 21, 64, 65, 150], "Q": [3, 70, 71, 129, 140], "R": [5, 64, 128, 200], "S": [1, 12, 66, 90],
-            "T": [2, 31, 64, 100]}[name]
+            "T": [2, 31, 64, 100], "U": [1, 7, 65, 80]}[name]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T", "U"])
 def test_whole_prompts(name, dtype):
     eng = engine(name, dtype)
     for i, n in enumerate(lengths(name)):
@@ -325,7 +326,7 @@ def test_prompt_then_token_by_token(name, head, n, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T", "U"])
 def test_unequal_batches_and_slots_used_again(name, dtype):
     """Requests of unequal lengths start together and are decoded together, the shorter ones ending earlier; then
     other requests take the slots and pages that came free (the cache has room for little more than one batch), in
