@@ -268,9 +268,12 @@ def test_trace_run_names_the_step_it_cannot_run(tmp_path):
     import sys
     from helpers import ROOT
     folder = model_folder("A")
-    for bad, reason in (([1] * 65, "CacheFull"), ([1, 10 ** 6], "vocabulary")):
+    # (the runner adds room for the partly filled last pages of at least 32 requests to --max-tokens: 40 requests of a
+    # whole page each are more than 64 tokens and that room)
+    too_many = [{"id": f"y{i}", "tokens": [1] * 64, "want": []} for i in range(40)]
+    for bad, reason in ((too_many, "CacheFull"), ([{"id": "y", "tokens": [1, 10 ** 6], "want": [0]}], "vocabulary")):
         steps = [{"step": 0, "entries": [{"id": "x", "tokens": [1, 2, 3], "want": [2]}], "end": ["x"]},
-                 {"step": 1, "entries": [{"id": "y", "tokens": bad, "want": [0]}], "end": []}]
+                 {"step": 1, "entries": bad, "end": []}]
         cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
                "--out", str(tmp_path / "o"), "--max-tokens", "64"]
         proc = subprocess.run(cmd, input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
