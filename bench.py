@@ -167,7 +167,7 @@ def through_generate(eng, cfg, batch, prompt_len, warmup, steps, weight_bytes, u
     return batch / step_s, step_s, step_bytes
 
 # ----------------------------------------------------------------------------- two designs side by side
-DESIGN_SIZES = {     # layers, width, heads, kv heads, head size, feed-forward, vocabulary
+SIDE_BY_SIDE_SIZES = {     # layers, width, heads, kv heads, head size, feed-forward, vocabulary
     "small": (4, 1024, 8, 8, 128, 4096, 32768),
     "mid": (4, 2048, 16, 8, 128, 8192, 32768),
     "large": (4, 4096, 32, 8, 128, 12288, 32768),
@@ -180,7 +180,7 @@ def design_configs(size, window, context):
     values of 128), two residual streams and a window that keeps 4 first keys."""
     from synaptix_amd import Qwen3Config
     from synaptix_amd.config import BizipelConfig
-    L, W, nh, nkv, hd, ff, V = DESIGN_SIZES[size]
+    L, W, nh, nkv, hd, ff, V = SIDE_BY_SIDE_SIZES[size]
     qwen = Qwen3Config.from_dict(dict(_COMMON, num_hidden_layers=L, hidden_size=W, num_attention_heads=nh,
                                       num_key_value_heads=nkv, head_dim=hd, intermediate_size=ff, vocab_size=V,
                                       tie_word_embeddings=True, max_position_embeddings=context))
@@ -201,8 +201,8 @@ def designs_side_by_side(args) -> int:
     from synaptix_amd.kernels import ops
     sizes = [s for s in args.sizes.split(",") if s]
     for s in sizes:
-        if s not in DESIGN_SIZES:
-            print(f"bench.py: --sizes names {s!r}; known: {', '.join(DESIGN_SIZES)}")
+        if s not in SIDE_BY_SIDE_SIZES:
+            print(f"bench.py: --sizes names {s!r}; known: {', '.join(SIDE_BY_SIDE_SIZES)}")
             return 2
     P, B = args.prompt, args.batch
     steps, warmup = (args.steps or 32), min(args.warmup, 8)
@@ -260,7 +260,7 @@ def designs_side_by_side(args) -> int:
             "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "ms_per_step": points[f"{first}_bizipel_decode_b{B}_ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
-            "config": {"model": "Bizipel beside Qwen3 at equal layer sizes", "sizes": {s: list(DESIGN_SIZES[s]) for s in sizes},
+            "config": {"model": "Bizipel beside Qwen3 at equal layer sizes", "sizes": {s: list(SIDE_BY_SIDE_SIZES[s]) for s in sizes},
                        "global_batch": B, "seq_len": P, "window": args.window, "parallelism": "single GPU",
                        "graph": not args.no_graph},
             "points": points}
