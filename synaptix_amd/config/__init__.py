@@ -1,8 +1,9 @@
 from .errors import ConfigError
 from .qwen3 import Qwen3Config
 from .bizipel import BizipelConfig
+from .kamivik import KamivikConfig
 from .registry import (Architecture, register_architecture, resolve_architecture, known_architectures,
                        load_config, read_config_json)
 
-__all__ = ["ConfigError", "Qwen3Config", "BizipelConfig", "Architecture", "register_architecture", "resolve_architecture",
+__all__ = ["ConfigError", "Qwen3Config", "BizipelConfig", "KamivikConfig", "Architecture", "register_architecture", "resolve_architecture",
            "known_architectures", "load_config", "read_config_json"]

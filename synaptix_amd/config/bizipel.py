@@ -19,29 +19,7 @@ from typing import Optional
 import numpy as np
 
 from .errors import ConfigError
-
-
-def _obj(d, key, where):
-    v = d.get(key) if isinstance(d, dict) else None
-    if not isinstance(v, dict):
-        raise ConfigError(f"{where}: {key!r} must be an object")
-    return v
-
-
-def _int(d, key, where, least=1):
-    v = d.get(key)
-    if isinstance(v, bool) or not isinstance(v, (int, float)) or int(v) != v:
-        raise ConfigError(f"{where}: {key!r} must be an integer, got {v!r}")
-    if int(v) < least:
-        raise ConfigError(f"{where}: {key!r} == {v} (must be at least {least})")
-    return int(v)
-
-
-def _num(d, key, where):
-    v = d.get(key)
-    if isinstance(v, bool) or not isinstance(v, (int, float)):
-        raise ConfigError(f"{where}: {key!r} must be a number, got {v!r}")
-    return float(v)
+from .fields import obj as _obj, integer as _int, number as _num
 
 
 @dataclass(frozen=True)

@@ -1,0 +1,308 @@
+// Products of rows with one of several weight matrices, chosen by the row's group:
+//
+//   out[orow(r), b, n] = epilogue( sum_k A[arow(r), b, k] * W[b, n, k] )         b: the group (an expert, a head)
+//
+// Two ways to say which rows meet which matrix:
+//   * segments: seg_start[b] <= r < seg_start[b + 1] are the rows of group b (tokens sorted by expert), with
+//     arow(r) = a_rows[r] and orow(r) = o_rows[r] gathered through index lists;
+//   * every group takes all M rows (a linear map for each head of a token): A, W and out move on by a fixed
+//     number of elements from one group to the next.
+// Epilogue, in this order and each optional: the exact GELU 0.5 z (1 + erf(z / sqrt 2)); a weight of the row;
+// sigmoid of a gate value read from float rows.  Sums are 32-bit.  bf16 operands whose K is a multiple of 32 run on
+// the matrix cores (16x16x32, operands straight from memory as 16-byte pieces of rows, no LDS: a wave computes 32
+// rows x 64 columns); everything else, and all of the 32-bit path, is plain FMA with one wave a (row, 8 columns).
+//
+// Beside it: the router of a mixture of experts (logits, the largest `top` of them, softmax over those) and the
+// counting sort that turns its choices into segments.
+#include "common.h"
+
+struct GroupedArgs {
+  const void* a;
+  long lda, a_group;        // A[row, group, k] = a[row * lda + group * a_group + k]
+  const void* w;
+  long w_group, ldw;        // W[group, n, k] = w[group * w_group + n * ldw + k]
+  void* out;
+  long ldo, o_group;        // out[row, group, n] = out[row * ldo + group * o_group + n]
+  int out_is_f32;
+  const int* seg_start;     // [groups + 1], or null: every group takes rows 0 .. M - 1
+  const int* a_rows;        // [rows] or null
+  const int* o_rows;        // [rows] or null
+  const float* row_weight;  // [rows] or null
+  const float* gate;        // or null: gate[row * gate_ld + group * gate_group + n * gate_col]
+  long gate_ld, gate_group;
+  int gate_col;
+  int act;                  // 0: none, 1: exact GELU
+  int M, N, K, groups;
+};
+
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+
+__device__ __forceinline__ float grouped_epilogue(const GroupedArgs& g, float v, int r, int b, int n) {
+  if (g.act == 1) v = gelu_erf(v);
+  if (g.row_weight) v *= g.row_weight[r];
+  if (g.gate) {
+    const float z = g.gate[(size_t)r * g.gate_ld + (size_t)b * g.gate_group + (size_t)n * g.gate_col];
+    v *= 1.f / (1.f + expf(-z));
+  }
+  return v;
+}
+
+__device__ __forceinline__ void grouped_store(const GroupedArgs& g, int r, int b, int n, float v) {
+  const int orow = g.o_rows ? g.o_rows[r] : r;
+  const size_t at = (size_t)orow * g.ldo + (size_t)b * g.o_group + n;
+  if (g.out_is_f32) ((float*)g.out)[at] = v;
+  else ((bf16*)g.out)[at] = (bf16)v;
+}
+
+// ---------------------------------------------------------------- plain FMA: one wave a (row, 8 columns)
+template <typename T>
+__global__ void __launch_bounds__(256) grouped_product_simt_kernel(GroupedArgs g) {
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  int r = blockIdx.x, b = blockIdx.z;
+  if (g.seg_start) {
+    // the group whose segment holds row r (segments are in order and cover 0 .. seg_start[groups] - 1)
+    if (r >= g.seg_start[g.groups]) return;
+    int lo = 0, hi = g.groups;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) / 2;
+      if (g.seg_start[mid] <= r) lo = mid; else hi = mid;
+    }
+    b = lo;
+  }
+  const int n0 = (blockIdx.y * 4 + wave) * 8;
+  if (n0 >= g.N) return;
+  const int arow = g.a_rows ? g.a_rows[r] : r;
+  const T* a = (const T*)g.a + (size_t)arow * g.lda + (size_t)b * g.a_group;
+  const T* w = (const T*)g.w + (size_t)b * g.w_group;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int k = lane; k < g.K; k += SYN_WAVE) {
+    const float x = to_f32<T>(a[k]);
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (n0 + c < g.N) acc[c] = fmaf(x, to_f32<T>(w[(size_t)(n0 + c) * g.ldw + k]), acc[c]);
+  }
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float v = wave_sum(acc[c]);
+    if (lane == 0 && n0 + c < g.N) grouped_store(g, r, b, n0 + c, grouped_epilogue(g, v, r, b, n0 + c));
+  }
+}
+
+// ---------------------------------------------------------------- bf16 on the matrix cores
+// D = W_tile (16 outputs x 32 k) . A_tile^T (32 k x 16 rows): a lane then holds four consecutive outputs of one row.
+// Both operands are 16-byte pieces of rows (8 k-values of lane group lane / 16), so whatever order the instruction
+// gives the k-values inside a lane group, the two operands agree.
+#define GP_TM 32
+__global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g) {
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, q = lane / 16;
+  int b = blockIdx.z, row0, row_end;
+  if (g.seg_start) {
+    int t = blockIdx.x;
+    b = -1;
+    for (int e = 0; e < g.groups; ++e) {
+      const int s0 = g.seg_start[e], n = g.seg_start[e + 1] - s0, tiles = (n + GP_TM - 1) / GP_TM;
+      if (t < tiles) {
+        b = e, row0 = s0 + t * GP_TM, row_end = s0 + n;
+        break;
+      }
+      t -= tiles;
+    }
+    if (b < 0) return;
+  } else {
+    row0 = blockIdx.x * GP_TM, row_end = g.M;
+    if (row0 >= row_end) return;
+  }
+  const int n0 = (blockIdx.y * 4 + wave) * 64;
+  if (n0 >= g.N) return;
+  const bf16* A = (const bf16*)g.a + (size_t)b * g.a_group;
+  const bf16* W = (const bf16*)g.w + (size_t)b * g.w_group;
+  const bf16* arow[2];
+  bool a_ok[2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int r = row0 + mb * 16 + i;
+    a_ok[mb] = r < row_end;
+    const int src = a_ok[mb] ? (g.a_rows ? g.a_rows[r] : r) : 0;
+    arow[mb] = A + (size_t)src * g.lda + q * 8;
+  }
+  const bf16* wrow[4];
+  bool w_ok[4];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const int n = n0 + nb * 16 + i;
+    w_ok[nb] = n < g.N;
+    wrow[nb] = W + (size_t)(w_ok[nb] ? n : 0) * g.ldw + q * 8;
+  }
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < g.K; k0 += 32) {
+    bf16x8 xa[2], xw[4];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) xa[mb] = a_ok[mb] ? *(const bf16x8*)(arow[mb] + k0) : zero;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) xw[nb] = w_ok[nb] ? *(const bf16x8*)(wrow[nb] + k0) : zero;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xw[nb], xa[mb], acc[mb][nb], 0, 0, 0);
+  }
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int r = row0 + mb * 16 + i;
+    if (r >= row_end) continue;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = n0 + nb * 16 + q * 4 + e;
+        if (n < g.N) grouped_store(g, r, b, n, grouped_epilogue(g, acc[mb][nb][e], r, b, n));
+      }
+  }
+}
+
+// rows_bound: with segments, the number of rows in all segments together (what the index lists hold)
+SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const void* w, long w_group, long ldw, void* out,
+                                   long ldo, long o_group, int in_is_f32, int out_is_f32, const int* seg_start,
+                                   const int* a_rows, const int* o_rows, const float* row_weight, const float* gate,
+                                   long gate_ld, long gate_group, int gate_col, int act, int M, int N, int K, int groups,
+                                   int rows_bound, int force_simt, hipStream_t stream) {
+  SYN_CHECK(M > 0 && N > 0 && K > 0 && groups > 0, "grouped_product: empty input (%d rows, %d x %d, %d groups)", M, N, K, groups);
+  SYN_CHECK(act == 0 || act == 1, "grouped_product: unknown activation code %d", act);
+  SYN_CHECK(seg_start != nullptr || (a_rows == nullptr && o_rows == nullptr && row_weight == nullptr),
+            "grouped_product: index lists and row weights come with segments");
+  SYN_CHECK(seg_start == nullptr || rows_bound > 0, "grouped_product: segments over %d rows", rows_bound);
+  SYN_CHECK(seg_start == nullptr || gate == nullptr, "grouped_product: a gate is read by row and group, not through segments");
+  const GroupedArgs g = {a, lda, a_group, w, w_group, ldw, out, ldo, o_group, out_is_f32, seg_start, a_rows, o_rows,
+                         row_weight, gate, gate_ld, gate_group, gate_col, act, M, N, K, groups};
+  const bool aligned = K % 32 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ldw % 8 == 0 && w_group % 8 == 0 &&
+                       (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+  if (!in_is_f32 && aligned && !force_simt) {
+    const int row_tiles = seg_start ? (rows_bound + GP_TM - 1) / GP_TM + groups : (M + GP_TM - 1) / GP_TM;
+    const dim3 grid(row_tiles, (N + 255) / 256, seg_start ? 1 : groups);
+    grouped_product_mfma_kernel<<<grid, 256, 0, stream>>>(g);
+  } else {
+    const dim3 grid(seg_start ? rows_bound : M, (N + 31) / 32, seg_start ? 1 : groups);
+    if (in_is_f32) grouped_product_simt_kernel<float><<<grid, 256, 0, stream>>>(g);
+    else grouped_product_simt_kernel<bf16><<<grid, 256, 0, stream>>>(g);
+  }
+  SYN_LAUNCH_CHECK("grouped_product");
+  return 0;
+}
+
+// ---------------------------------------------------------------- router: logits, the largest `top`, their softmax
+// One workgroup a token.  z[e] = sum_k x[k] W[e, k] + bias[e] in 32-bit; of equal logits the lower index comes first.
+#define ROUTE_MAX_EXPERTS 1024
+#define ROUTE_MAX_TOP 64
+template <typename T>
+__global__ void __launch_bounds__(256) route_topk_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                         const float* __restrict__ bias, int* __restrict__ ids,
+                                                         float* __restrict__ weights, int H, int E, int top) {
+  __shared__ float z[ROUTE_MAX_EXPERTS];
+  __shared__ float chosen[ROUTE_MAX_TOP];
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, tok = blockIdx.x;
+  const T* xr = x + (size_t)tok * H;
+  for (int e = wave; e < E; e += 4) {
+    const T* wr = w + (size_t)e * H;
+    float acc = 0.f;
+    for (int k = lane; k < H; k += SYN_WAVE) acc = fmaf(to_f32<T>(xr[k]), to_f32<T>(wr[k]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc + (bias ? bias[e] : 0.f);
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  for (int t = 0; t < top; ++t) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += SYN_WAVE) {
+      const float v = z[e];
+      if (v > best) best = v, at = e;      // (a lane meets its experts in rising order)
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, SYN_WAVE);
+      const int oa = __shfl_xor(at, off, SYN_WAVE);
+      if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+    }
+    if (lane == 0) {
+      if (at >= E) at = t;          // every logit left is NaN or -inf: any expert, and no access beyond the table
+      ids[(size_t)tok * top + t] = at;
+      chosen[t] = best;
+      z[at] = -INFINITY;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (lane == 0) {
+    const float m = chosen[0];      // the first chosen is the largest
+    float sum = 0.f;
+    for (int t = 0; t < top; ++t) sum += expf(chosen[t] - m);
+    for (int t = 0; t < top; ++t) weights[(size_t)tok * top + t] = expf(chosen[t] - m) / sum;
+  }
+}
+
+SYN_EXPORT int syn_route_topk(const void* x, const void* w, int is_f32, const float* bias, int* ids, float* weights,
+                              int n_tokens, int H, int E, int top, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && H > 0, "route_topk: empty input");
+  SYN_CHECK(E > 0 && E <= ROUTE_MAX_EXPERTS, "route_topk: %d experts (at most %d)", E, ROUTE_MAX_EXPERTS);
+  SYN_CHECK(top > 0 && top <= E && top <= ROUTE_MAX_TOP, "route_topk: the %d largest of %d (at most %d)", top, E, ROUTE_MAX_TOP);
+  if (is_f32)
+    route_topk_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)x, (const float*)w, bias, ids, weights, H, E, top);
+  else
+    route_topk_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, bias, ids, weights, H, E, top);
+  SYN_LAUNCH_CHECK("route_topk");
+  return 0;
+}
+
+// ---------------------------------------------------------------- the router's choices as segments
+// P = n_tokens * top pairs (token n, its t-th expert), pair p = n * top + t.  Sorted by expert:
+//   seg_start[e] .. seg_start[e + 1]: the places of expert e;  for a place r:
+//   tok_of[r] = n, pair_of[r] = p, part_of[r] = t * n_tokens + n (the pair's row in partial sums [top, n_tokens]),
+//   weight_of[r] = weights[p].
+// One workgroup.  The order inside a segment is the order of arrival; no result depends on it (a row's sums do not
+// depend on its place in a tile).
+__global__ void __launch_bounds__(1024) route_sort_kernel(const int* __restrict__ ids, const float* __restrict__ weights,
+                                                          int* __restrict__ seg_start, int* __restrict__ tok_of,
+                                                          int* __restrict__ pair_of, int* __restrict__ part_of,
+                                                          float* __restrict__ weight_of, int n_tokens, int top, int E) {
+  __shared__ int count[ROUTE_MAX_EXPERTS];
+  __shared__ int cursor[ROUTE_MAX_EXPERTS];
+  const int P = n_tokens * top;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[min(max(ids[p], 0), E - 1)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      cursor[e] = at;
+      seg_start[e] = at;
+      at += count[e];
+    }
+    seg_start[E] = at;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int r = atomicAdd(&cursor[min(max(ids[p], 0), E - 1)], 1);
+    const int n = p / top, t = p % top;
+    tok_of[r] = n;
+    pair_of[r] = p;
+    part_of[r] = t * n_tokens + n;
+    weight_of[r] = weights[p];
+  }
+}
+
+SYN_EXPORT int syn_route_sort(const int* ids, const float* weights, int* seg_start, int* tok_of, int* pair_of,
+                              int* part_of, float* weight_of, int n_tokens, int top, int E, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && top > 0, "route_sort: empty input");
+  SYN_CHECK(E > 0 && E <= ROUTE_MAX_EXPERTS, "route_sort: %d experts (at most %d)", E, ROUTE_MAX_EXPERTS);
+  SYN_CHECK((long)n_tokens * top < (1L << 30), "route_sort: %d tokens x %d", n_tokens, top);
+  route_sort_kernel<<<1, 1024, 0, stream>>>(ids, weights, seg_start, tok_of, pair_of, part_of, weight_of, n_tokens, top, E);
+  SYN_LAUNCH_CHECK("route_sort");
+  return 0;
+}

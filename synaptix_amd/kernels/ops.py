@@ -1058,3 +1058,183 @@ def measure_ceilings(device="cuda:0", read_bytes=1 << 30, repeats=5):
     t_mfma = best(lambda: _call(lib, "syn_probe_mfma", groups, iters, _ptr(fsink), _stream()))
     flops = groups * 4 * iters * 4 * 2 * 32 * 32 * 16
     return buf.numel() * 4 / t_read / 1e9, flops / t_mfma / 1e12
+
+
+# ----------------------------------------------------------------------------- scaled residual terms
+
+def add_scaled_rmsnorm(resid, terms, gain, eps, out, rows=None):
+    """resid += sum_t scale_t * delta_t for up to two terms (delta float [N, H] or partial sums [S, N, H], scale float
+    [H] or None), then out = RMSNorm(resid) * gain when `out` is given.  rows [n] int32: only those rows are summed and
+    normed, resid is not written."""
+    _need(resid, "add_scaled_rmsnorm.resid", _F32, (None, None))
+    N, H = resid.shape
+    if not 1 <= len(terms) <= 2:
+        raise KernelError(f"add_scaled_rmsnorm: {len(terms)} terms (one or two)")
+    args = []
+    for i, (d, s) in enumerate(terms):
+        parts = d.shape[0] if d.dim() == 3 else 1
+        _need(d, f"add_scaled_rmsnorm.delta{i}", _F32, (parts, N, H) if d.dim() == 3 else (N, H))
+        if s is not None:
+            _need(s, f"add_scaled_rmsnorm.scale{i}", _F32, (H,))
+        args += [_ptr(d), parts, _ptr(s)]
+    if len(terms) == 1:
+        args += [_ptr(None), 1, _ptr(None)]
+    n_out = N
+    if rows is not None:
+        _need(rows, "add_scaled_rmsnorm.rows", _I32, (None,))
+        n_out = rows.shape[0]
+    if out is not None:
+        _need(gain, "add_scaled_rmsnorm.gain", (_BF16, _F32), (H,))
+        _need(out, "add_scaled_rmsnorm.out", (_BF16, _F32), (n_out, H))
+    elif rows is not None:
+        raise KernelError("add_scaled_rmsnorm: gathered rows without an output")
+    _call(load_library("core"), "syn_add_scaled_rmsnorm", _ptr(resid), N, _ptr(rows), n_out, *args, _ptr(gain),
+          0 if gain is None else _is_f32(gain), ctypes.c_float(eps), _ptr(out), 0 if out is None else _is_f32(out), H,
+          _stream())
+
+
+# ----------------------------------------------------------------------------- products by group (experts, heads)
+
+def _grouped(name, a, lda, a_group, w, w_group, ldw, out, ldo, o_group, M, N, K, groups, seg=None, a_rows=None,
+             o_rows=None, row_weight=None, gate=None, gate_ld=0, gate_group=0, gate_col=0, act=0, rows_bound=0,
+             force_simt=False):
+    L = ctypes.c_long
+    _call(load_library("core"), "syn_grouped_product", _ptr(a), L(lda), L(a_group), _ptr(w), L(w_group), L(ldw), _ptr(out),
+          L(ldo), L(o_group), _is_f32(a), _is_f32(out), _ptr(seg), _ptr(a_rows), _ptr(o_rows), _ptr(row_weight), _ptr(gate),
+          L(gate_ld), L(gate_group), int(gate_col), int(act), int(M), int(N), int(K), int(groups), int(rows_bound),
+          int(bool(force_simt)), _stream())
+
+
+def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force_simt=False):
+    """A linear map for each head:  out[n, h, out_offset + j] = sum_k x[n, h, k] * w[h, j, k]  [* sigmoid(gate)].
+    x [N, heads, K] and w [heads, J, K] in the engine's type, out [N, heads, >= out_offset + J] in that type.
+    gate: float rows (columns of a fused projection, any row stride) that hold heads * J values (one for each output,
+    gate_per_value) or `heads` values (one a head)."""
+    _need(x, "heads_product.x", (_BF16, _F32), (None, None, None))
+    N, Hn, K = x.shape
+    _need(w, "heads_product.w", x.dtype, (Hn, None, K))
+    J = w.shape[1]
+    _need(out, "heads_product.out", x.dtype, (N, Hn, None))
+    Jo = out.shape[2]
+    if out_offset < 0 or out_offset + J > Jo:
+        raise KernelError(f"heads_product: {J} outputs at {out_offset} do not fit rows of {Jo}")
+    kw = {}
+    if gate is not None:
+        need = Hn * J if gate_per_value else Hn
+        kw = dict(gate=gate, gate_ld=_float_rows_view(gate, "heads_product.gate", N, need),
+                  gate_group=J if gate_per_value else 1, gate_col=1 if gate_per_value else 0)
+    if out_offset:
+        out = out.view(-1)[out_offset:]
+    _grouped("heads_product", x, Hn * K, K, w, J * K, K, out, Hn * Jo, Jo, N, J, K, Hn, force_simt=force_simt, **kw)
+
+
+ROUTE_MAX_EXPERTS, ROUTE_MAX_TOP = 1024, 64
+
+
+def route_topk(x, w, bias, ids, weights):
+    """Router of a mixture of experts: z = x . w^T + bias in 32-bit; ids [N, top] int32 the experts with the largest
+    logits (largest first, the lower index of equal ones), weights [N, top] float the softmax over those logits."""
+    _need(x, "route_topk.x", (_BF16, _F32), (None, None))
+    N, H = x.shape
+    _need(w, "route_topk.w", x.dtype, (None, H))
+    E = w.shape[0]
+    if bias is not None:
+        _need(bias, "route_topk.bias", _F32, (E,))
+    _need(ids, "route_topk.ids", _I32, (N, None))
+    top = ids.shape[1]
+    _need(weights, "route_topk.weights", _F32, (N, top))
+    if not (0 < top <= min(E, ROUTE_MAX_TOP)) or E > ROUTE_MAX_EXPERTS:
+        raise KernelError(f"route_topk: the {top} largest of {E} experts (at most {ROUTE_MAX_TOP} of {ROUTE_MAX_EXPERTS})")
+    _call(load_library("core"), "syn_route_topk", _ptr(x), _ptr(w), _is_f32(x), _ptr(bias), _ptr(ids), _ptr(weights), N, H,
+          E, top, _stream())
+
+
+def route_sort(ids, weights, n_experts):
+    """The router's choices sorted by expert.  Returns (seg_start [E + 1], tok_of, pair_of, part_of int32 [N * top],
+    weight_of float [N * top]): the places seg_start[e] .. seg_start[e + 1] belong to expert e; a place holds the token,
+    the pair n * top + t, the pair's row t * N + n in partial sums [top, N], and the pair's weight."""
+    _need(ids, "route_sort.ids", _I32, (None, None))
+    N, top = ids.shape
+    _need(weights, "route_sort.weights", _F32, (N, top))
+    if not 0 < n_experts <= ROUTE_MAX_EXPERTS:
+        raise KernelError(f"route_sort: {n_experts} experts (at most {ROUTE_MAX_EXPERTS})")
+    lists = torch.empty((3, N * top), dtype=_I32, device=ids.device)
+    seg = torch.empty(n_experts + 1, dtype=_I32, device=ids.device)
+    weight_of = torch.empty(N * top, dtype=_F32, device=ids.device)
+    _call(load_library("core"), "syn_route_sort", _ptr(ids), _ptr(weights), _ptr(seg), _ptr(lists[0]), _ptr(lists[1]),
+          _ptr(lists[2]), _ptr(weight_of), N, top, n_experts, _stream())
+    return seg, lists[0], lists[1], lists[2], weight_of
+
+
+def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False, force_simt=False):
+    """out[o_rows[r]] = epilogue(x[a_rows[r]] . w[e]^T) for the places r of each expert e's segment.  x [*, K] in the
+    engine's type, w [E, J, K] in that type, out [*, J] in that type or float; the index lists come from route_sort and
+    must stay inside x and out (the caller's contract: they are on the device).  Epilogue: the exact GELU, then the
+    row's weight, each if asked for."""
+    _need(x, "experts_product.x", (_BF16, _F32), (None, None))
+    K = x.shape[1]
+    _need(w, "experts_product.w", x.dtype, (None, None, K))
+    E, J = w.shape[0], w.shape[1]
+    _need(out, "experts_product.out", (x.dtype, _F32), (None, J))
+    _need(seg, "experts_product.seg", _I32, (E + 1,))
+    _need(a_rows, "experts_product.a_rows", _I32, (None,))
+    P = a_rows.shape[0]
+    _need(o_rows, "experts_product.o_rows", _I32, (P,))
+    if row_weight is not None:
+        _need(row_weight, "experts_product.row_weight", _F32, (P,))
+    _grouped("experts_product", x, K, 0, w, J * K, K, out, J, 0, P, J, K, E, seg=seg, a_rows=a_rows, o_rows=o_rows,
+             row_weight=row_weight, act=1 if gelu else 0, rows_bound=P, force_simt=force_simt)
+
+
+# ----------------------------------------------------------------------------- latent attention: intake
+
+def latent_intake(proj, gain, eps, cos, sin, q_nope, q_full, k_pages, v_pages, page_table, tok_seq, tok_pos,
+                  n_heads, dim, rot_dim, rank, max_position, write_kv=True):
+    """From the fused projection proj [N, >= heads * (dim + rot_dim) + rank + rot_dim] float: q_nope [N, heads * dim];
+    the rotated query parts into q_full [N, heads * (rank + rot_dim)] behind each head's first `rank` places; the
+    token's cache row [RMSNorm(latent) * gain | rotated key part] into k_pages [pages, 1, 64, rank + rot_dim] and the
+    normed latent as its value into v_pages [pages, 1, rank, 64].  cos, sin [capacity, pairs]: pairs (2i, 2i + 1) of
+    the rotated parts are turned, what lies behind 2 * pairs passes."""
+    _need(proj, "latent_intake.proj", _F32, (None, None))
+    N, width = proj.shape
+    R = rank + rot_dim
+    if width < n_heads * (dim + rot_dim) + R:
+        raise KernelError(f"latent_intake: rows of {width} values do not hold {n_heads} queries and the latent")
+    _need(gain, "latent_intake.gain", (_BF16, _F32), (rank,))
+    n_pairs, capacity = 0, 0
+    if cos is not None:
+        _need(cos, "latent_intake.cos", _F32, (None, None))
+        capacity, n_pairs = cos.shape
+        _need(sin, "latent_intake.sin", _F32, (capacity, n_pairs))
+        if 2 * n_pairs > rot_dim or max_position >= capacity:
+            raise KernelError(f"latent_intake: {n_pairs} pairs in {rot_dim} values, position {max_position} of {capacity}")
+    _need(q_nope, "latent_intake.q_nope", (_BF16, _F32), (N, n_heads * dim))
+    _need(q_full, "latent_intake.q_full", q_nope.dtype, (N, n_heads * R))
+    _need(k_pages, "latent_intake.k_pages", q_nope.dtype, (None, 1, PAGE_TOKENS, R))
+    _need(v_pages, "latent_intake.v_pages", q_nope.dtype, (k_pages.shape[0], 1, rank, PAGE_TOKENS))
+    _need(page_table, "latent_intake.page_table", _I32, (None, None))
+    _need(tok_seq, "latent_intake.tok_seq", _I32, (N,))
+    _need(tok_pos, "latent_intake.tok_pos", _I32, (N,))
+    _call(load_library("core"), "syn_latent_intake", _ptr(proj), width, _ptr(gain), _is_f32(gain), ctypes.c_float(eps),
+          _ptr(cos), _ptr(sin), n_pairs, capacity, int(max_position), _ptr(q_nope), _ptr(q_full), _ptr(k_pages),
+          _ptr(v_pages), _is_f32(q_nope), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), N, n_heads,
+          dim, rot_dim, rank, int(bool(write_kv)), _stream())
+
+
+# ----------------------------------------------------------------------------- latent attention
+
+LATENT_ATTENTION_MAX_ROW = WINDOW_ATTENTION_MAX_DIM
+
+
+def latent_attention_takes(rank, rot_dim) -> bool:
+    return 0 < rank and rank + rot_dim <= LATENT_ATTENTION_MAX_ROW
+
+
+def latent_attention(q_full, k_pages, v_pages, page_table, ctx, out, scale, n_heads, rank, rot_dim, window=0):
+    """Attention of `n_heads` queries a token over one shared key row a cached token: q_full [N, heads * (rank +
+    rot_dim)], key rows k_pages [pages, 1, 64, rank + rot_dim] whose first `rank` values are the row's value (v_pages
+    [pages, 1, rank, 64] holds them once more, along the keys); out [N, heads * rank] = sum_j softmax_j(scale q . k_j)
+    k_j[:rank] over the keys at or before the query (window > 0: the last `window` of them).  ctx: the step's arrays
+    (tok_seq, tok_pos)."""
+    window_attention(q_full, k_pages, v_pages, page_table, ctx.tok_seq, ctx.tok_pos, out, scale, n_heads, 1, rank + rot_dim,
+                     rank, window=window)

@@ -143,3 +143,62 @@ class HyperConnectionBlock(Block):
             h2 = self._read(self.norm2, resid, self.hc[1][0], ctx.act_dtype, pending)
             pending = StreamsWrite(resid, self.hc[1][2], self.hc[1][1], self.feed_forward.forward(h2, ctx))
         return pending
+
+
+class ParallelBlock(Block):
+    """A layer whose mixer and feed-forward run side by side on the output of one norm:
+
+        h = norm(x);   x <- x + mult * (scale1 * mixer(h) + scale2 * ff(h))
+
+    with a scale for every channel of each sublayer's result (tensors prefix + "ls1", "ls2", [hidden]; `layer_scale`
+    False: none) and one factor `mult`.  A layer may have no feed-forward.  The sum is left to whoever reads the
+    residual next (parts.linear.ChannelScaledDeltas): a norm that takes it adds and norms in one pass."""
+    takes_deferred_product = True       # `pending` may be the ChannelScaledDeltas that the block before left
+
+    def __init__(self, prefix: str, hidden: int, norm, mixer, feed_forward=None, mult: float = 1.0,
+                 layer_scale: bool = True, scale_names=("ls1", "ls2")):
+        self.prefix, self.hidden, self.mult = prefix, hidden, float(mult)
+        self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+        self.layer_scale, self.scale_names = bool(layer_scale), tuple(scale_names)
+        self.scales = [None, None]
+
+    def _parts(self):
+        return [p for p in (self.norm, self.mixer, self.feed_forward) if p is not None]
+
+    @property
+    def capturable(self):
+        return all(getattr(p, "capturable", False) for p in self._parts())
+
+    def _scale_names(self):
+        n = 2 if self.feed_forward is not None else 1
+        return [self.prefix + s for s in self.scale_names[:n]] if self.layer_scale else []
+
+    def tensor_specs(self):
+        from ..weights.source import TensorSpec
+        specs = {}
+        for p in self._parts():
+            specs.update(p.tensor_specs())
+        specs.update({n: TensorSpec((self.hidden,), "gain") for n in self._scale_names()})
+        return specs
+
+    def load(self, get):
+        import torch
+        for p in self._parts():
+            p.load(get)
+        for i, n in enumerate(self._scale_names()):
+            self.scales[i] = (get(n).float() * self.mult).contiguous()       # mult * scale, 32-bit
+        if not self.layer_scale and self.mult != 1.0:
+            dev = self.norm.gain.device
+            self.scales = [torch.full((self.hidden,), self.mult, dtype=torch.float32, device=dev)] * 2
+
+    def check(self, dtype):
+        for p in self._parts():
+            p.check(dtype)
+
+    def forward(self, resid, pending, ctx, cache, owner=True):
+        from .linear import ChannelScaledDeltas
+        h = as_rows(self.norm.add_apply(resid, _norm_input(self.norm, pending), ctx.act_dtype))
+        terms = [(as_delta(self.mixer.forward(h, ctx, cache, owner)), self.scales[0])]
+        if self.feed_forward is not None:
+            terms.append((as_delta(self.feed_forward.forward(h, ctx)), self.scales[1]))
+        return ChannelScaledDeltas(terms)

@@ -70,3 +70,65 @@ class GatedMlp(FeedForward):
             h = as_rows(h)
             ops.swiglu(linear(h, self.w_gate_up, h.dtype), m, self.activation)
         return deferred_product(m, self.w_down)
+
+
+class RoutedExperts(FeedForward):
+    """A mixture of small ungated experts: each token goes through the `top` experts whose router logits are largest,
+
+        z = W_router h + b (32-bit);   chosen: the `top` largest z;   weights: softmax over the chosen logits only
+        y = sum_chosen weight_e * W_down[e] act(W_up[e] h)
+
+    The tokens are sorted by expert on the device (no count comes back to the host), and each expert's rows meet its
+    matrices in one launch for all experts (ops.experts_product).  Returns the `top` weighted results of every token
+    as partial sums [top, N, hidden], which whoever adds the residual sums up.
+    Tensors: prefix + "e<j>.up" [ff, hidden], "e<j>.down" [hidden, ff], "router" [experts, hidden], "router.b"."""
+    takes_scaled_rows = False
+    capturable = True
+
+    ACTIVATIONS = ("gelu",)       # the exact (erf) form, the products' epilogue
+
+    def __init__(self, prefix: str, hidden: int, ff: int, n_experts: int, top: int, activation: str = "gelu",
+                 router_bias: bool = True, names=("e{}.up", "e{}.down", "router", "router.b")):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"{prefix}: activation {activation!r} (the experts' products apply {self.ACTIVATIONS})")
+        if not 0 < top <= n_experts:
+            raise ValueError(f"{prefix}: the {top} largest of {n_experts} experts")
+        self.prefix, self.hidden, self.ff, self.n_experts, self.top = prefix, hidden, ff, n_experts, top
+        self.router_bias, self.names = bool(router_bias), tuple(names)
+        self.w_up = self.w_down = self.w_router = self.b_router = None
+
+    def tensor_specs(self):
+        p, (up, down, router, bias) = self.prefix, self.names
+        specs = {p + router: TensorSpec((self.n_experts, self.hidden))}
+        if self.router_bias:
+            specs[p + bias] = TensorSpec((self.n_experts,), "bias")
+        for e in range(self.n_experts):
+            specs[p + up.format(e)] = TensorSpec((self.ff, self.hidden))
+            specs[p + down.format(e)] = TensorSpec((self.hidden, self.ff))
+        return specs
+
+    def load(self, get):
+        p, (up, down, router, bias) = self.prefix, self.names
+        self.w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
+        self.w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
+        self.w_router = get(p + router)
+        self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
+
+    def check(self, dtype):
+        if self.n_experts > ops.ROUTE_MAX_EXPERTS or self.top > ops.ROUTE_MAX_TOP:
+            raise ValueError(f"{self.prefix}: {self.top} of {self.n_experts} experts "
+                             f"(at most {ops.ROUTE_MAX_TOP} of {ops.ROUTE_MAX_EXPERTS})")
+
+    def forward(self, h, ctx):
+        h = as_rows(h)
+        N, dev = h.shape[0], h.device
+        ids = torch.empty((N, self.top), dtype=torch.int32, device=dev)
+        weights = torch.empty((N, self.top), dtype=torch.float32, device=dev)
+        ops.route_topk(h, self.w_router, self.b_router, ids, weights)
+        seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, self.n_experts)
+        mid = torch.empty((N * self.top, self.ff), dtype=h.dtype, device=dev)
+        ops.experts_product(h, self.w_up, mid, seg, tok_of, pair_of, gelu=True)
+        y = torch.empty((self.top, N, self.hidden), dtype=torch.float32, device=dev)
+        ops.experts_product(mid, self.w_down, y.view(self.top * N, self.hidden), seg, pair_of, part_of,
+                            row_weight=weight_of)
+        return y

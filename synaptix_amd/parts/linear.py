@@ -123,9 +123,26 @@ class StreamsWrite:
         return out
 
 
+class ChannelScaledDeltas:
+    """The results of one or two sublayers that ran side by side, not yet added to the residual:
+    sum_i scale_i * term_i, each term a float tensor [N, hidden] or partial sums [P, N, hidden], each scale float
+    [hidden] (one factor for every channel) or None.  A norm that takes it (RmsNorm) adds the terms into the residual
+    and norms the rows in the same pass; everything else asks for `run()`, the sum as one tensor."""
+
+    def __init__(self, terms):
+        self.terms = [(as_delta(t), s) for t, s in terms]
+        self.shape = tuple(self.terms[0][0].shape[-2:])
+
+    def run(self):
+        first = self.terms[0][0]
+        total = torch.zeros(self.shape, dtype=torch.float32, device=first.device)
+        ops.add_scaled_rmsnorm(total, self.terms, None, 0.0, None)
+        return total
+
+
 def as_delta(d):
     """The delta of the residual rows as a tensor (or None), whatever form it arrives in."""
-    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas, StreamsWrite)) else d
+    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas, StreamsWrite, ChannelScaledDeltas)) else d
 
 
 def deferred_product(x, w):

@@ -13,7 +13,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import DeferredProduct, ScaledRows
+from .linear import DeferredProduct, ScaledRows, ChannelScaledDeltas
 
 
 class RmsNorm(Part):
@@ -38,6 +38,14 @@ class RmsNorm(Part):
     def add_apply(self, resid, delta, out_dtype, rows=None):
         """resid [N, dim] float: with rows None, resid += delta (if any) in place and every row is
         normed; with rows [n] int32 only those rows of resid + delta are normed and resid is kept."""
+        if isinstance(delta, ChannelScaledDeltas):
+            # the results of sublayers that ran side by side, each with its channels' scales: added and normed in one pass
+            if self.gain_offset == 0.0:
+                n = resid.shape[0] if rows is None else rows.shape[0]
+                out = torch.empty((n, self.dim), dtype=out_dtype, device=resid.device)
+                ops.add_scaled_rmsnorm(resid, delta.terms, self.gain, self.eps, out, rows)
+                return out
+            delta = delta.run()
         if isinstance(delta, DeferredProduct):
             # a product over packed weights for few rows: it adds its sums into resid itself and leaves the rows with
             # the gain and the row statistic in groups; the product that follows applies the row's factor

@@ -87,3 +87,34 @@ class LogDistanceBias(Position):
         if n_heads != self.n_heads:
             raise ValueError(f"a distance bias for {self.n_heads} heads was asked for {n_heads}")
         return self.r1, self.r2
+
+
+class RotaryInterleaved(Position):
+    """A rotation of the pairs (2i, 2i + 1), i < dims / 2, of a vector's first `dims` values by the angle
+    position * base^(-2i / dims); what lies behind `dims` passes unchanged.  The pair (u, v) becomes
+    (u cos a - v sin a, v cos a + u sin a).  Tables [capacity, dims / 2] are made on the host with 64-bit angles and
+    kept in 32-bit, once for all parts with the same constants."""
+    capturable = True
+    _shared: dict = {}
+
+    def __init__(self, base: float, dims: int, capacity: int):
+        if dims < 0 or dims % 2:
+            raise ValueError(f"rotated dims {dims} must be even and not negative")
+        if capacity <= 0:
+            raise ValueError("capacity must be positive")
+        self.base, self.dims, self.capacity = float(base), int(dims), int(capacity)
+
+    def host_tables(self):
+        half = self.dims // 2
+        freqs = np.power(np.float64(self.base), -2.0 * np.arange(half, dtype=np.float64) / max(self.dims, 1))
+        ang = np.arange(self.capacity, dtype=np.float64)[:, None] * freqs[None, :]
+        return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+    def tables(self, device):
+        if self.dims == 0:
+            return None, None
+        key = (self.base, self.dims, self.capacity, str(device))
+        if key not in self._shared:
+            cos, sin = self.host_tables()
+            self._shared[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))
+        return self._shared[key]
