@@ -1169,7 +1169,7 @@ def route_sort(ids, weights, n_experts):
 def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False, force_simt=False):
     """out[o_rows[r]] = epilogue(x[a_rows[r]] . w[e]^T) for the places r of each expert e's segment.  x [*, K] in the
     engine's type, w [E, J, K] in that type, out [*, J] in that type or float; the index lists come from route_sort and
-    must stay inside x and out (the caller's contract: they are on the device).  Epilogue: the exact GELU, then the
+    must stay inside x and out (the caller sees to that: they are on the device).  Epilogue: the exact GELU, then the
     row's weight, each if asked for."""
     _need(x, "experts_product.x", (_BF16, _F32), (None, None))
     K = x.shape[1]
@@ -1230,11 +1230,11 @@ def latent_attention_takes(rank, rot_dim) -> bool:
     return 0 < rank and rank + rot_dim <= LATENT_ATTENTION_MAX_ROW
 
 
-def latent_attention(q_full, k_pages, v_pages, page_table, ctx, out, scale, n_heads, rank, rot_dim, window=0):
+def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, rank, rot_dim, window=0):
     """Attention of `n_heads` queries a token over one shared key row a cached token: q_full [N, heads * (rank +
     rot_dim)], key rows k_pages [pages, 1, 64, rank + rot_dim] whose first `rank` values are the row's value (v_pages
     [pages, 1, rank, 64] holds them once more, along the keys); out [N, heads * rank] = sum_j softmax_j(scale q . k_j)
-    k_j[:rank] over the keys at or before the query (window > 0: the last `window` of them).  ctx: the step's arrays
-    (tok_seq, tok_pos)."""
-    window_attention(q_full, k_pages, v_pages, page_table, ctx.tok_seq, ctx.tok_pos, out, scale, n_heads, 1, rank + rot_dim,
+    k_j[:rank] over the keys at or before the query's position (window > 0: the last `window` of them).  Scores,
+    weights and sums are 32-bit."""
+    window_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, 1, rank + rot_dim,
                      rank, window=window)

@@ -107,7 +107,7 @@ class LatentAttention(Mixer):
         # the query in the latent's space, into the first `rank` places of each head's row
         ops.heads_product(q_nope.view(N, nh, dim), self.w_uk_t, q_full.view(N, nh, R))
         o_lat = torch.empty((N, nh * rank), dtype=act, device=dev)
-        ops.latent_attention(q_full, cache.k_pages, cache.v_pages, table, ctx, o_lat, self.scale, nh, rank, rot,
+        ops.latent_attention(q_full, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o_lat, self.scale, nh, rank, rot,
                              window=self.window or 0)
         o = torch.empty((N, nh * vdim), dtype=act, device=dev)
         gate = proj[:, nh * (dim + rot) + R:] if self.gate else None
