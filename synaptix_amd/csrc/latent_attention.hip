@@ -1,0 +1,262 @@
+// Latent attention in bf16 on the matrix cores: every head's query against ONE key row a cached token.
+//
+//   q       [N][heads][R]        R = rank + rot: the query in the latent's space, then its rotated part
+//   k_pages [pages][64][R]       a token's row [latent | rotated key part]
+//   v_pages [pages][rank][64]    the latent once more, along the keys
+//   out     [N][heads][rank]     sum_j softmax_j(scale q . k_j) k_j[:rank]  over the keys j that the query sees:
+//                                j <= position, and position - j < window if there is a window
+//
+// Since all heads share the keys, the 16 rows of a tile are 16 consecutive (token, head) pairs of one sequence: for
+// a single token its heads (decoding is a small matrix product, not a matrix-vector one), for a prompt a few tokens
+// with all their heads.  One wave a tile, no LDS:
+//   S^T (keys x rows)  = K (16 keys x k) . Q^T (k x 16 rows)        a lane holds four keys of ONE row
+//   O^T (rank x rows) += V^T (16 values x 32 keys) . P^T (32 keys x 16 rows)
+// and what a lane holds of S^T is exactly its share of the operand P^T (the 32 keys of a k-step are taken in the
+// order in which two score tiles leave them, and V^T's 8-byte pieces are fetched in that order too).  The scores
+// and weights are 32-bit; a weight meets V as two bf16 numbers (the weight rounded, and what the rounding left), so
+// it counts with 16 bits of mantissa although the product runs in bf16; sums are 32-bit.
+// A tile's pages may be cut into splits (grid y) whose partial results a second kernel merges: single tokens over
+// long sequences then fill the chip.
+#include "common.h"
+
+#define LA_ROWS 16
+
+template <bool X32> struct LaFrag;
+template <> struct LaFrag<false> { typedef bf16x4 type; };
+template <> struct LaFrag<true> { typedef bf16x8 type; };
+
+__device__ __forceinline__ f32x4 la_mfma(bf16x4 a, bf16x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 la_mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// the sequence and the tile inside it of global tile t; false: beyond the last tile
+__device__ __forceinline__ bool la_find_tile(int t, const int* seq_start, int n_seqs, int nh, int& seq, int& tile,
+                                             int& start, int& rows) {
+  for (int b = 0; b < n_seqs; ++b) {
+    const int s0 = seq_start[b], n = (seq_start[b + 1] - s0) * nh, tiles = (n + LA_ROWS - 1) / LA_ROWS;
+    if (t < tiles) {
+      seq = b, tile = t, start = s0, rows = n;
+      return true;
+    }
+    t -= tiles;
+  }
+  return false;
+}
+
+// DT: tiles of 16 values that the accumulators hold (rank <= 16 DT); QS: k-steps that the query's registers hold
+// (R <= QS * (X32 ? 32 : 16)); X32: k-steps of 32 (R a multiple of 32) or of 16.
+template <int DT, int QS, bool X32>
+__global__ void __launch_bounds__(256)
+latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+                             const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
+                             const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out,
+                             float* __restrict__ part_o, float* __restrict__ part_ml, float scale, int nh, int rank, int R,
+                             int window, int n_splits) {
+  typedef typename LaFrag<X32>::type frag;
+  constexpr int KS = X32 ? 32 : 16, PIECE = KS / 4;
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, g = lane / 16;
+  const int gt = blockIdx.x * 4 + wave, split = blockIdx.y;
+  int seq, tile, start, rows;
+  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;      // (no barrier anywhere below)
+  const int past = seq_past[seq];
+  const int flat0 = tile * LA_ROWS, flat_last = min(flat0 + LA_ROWS, rows) - 1;
+  const bool row_ok = flat0 + i < rows;
+  const int flat = row_ok ? flat0 + i : flat_last;       // a row beyond the tile's end repeats the last one, unstored
+  const int tok = flat / nh, head = flat % nh, pos = past + tok;
+  const int kv_len = past + rows / nh;
+  // the pages that some row of the tile sees, and this split's share of them
+  const int pos_lo = past + flat0 / nh, pos_hi = past + flat_last / nh;
+  const int key_lo = window > 0 ? max(0, pos_lo - window + 1) : 0;
+  const int page_lo = key_lo / SYN_PAGE, page_hi = pos_hi / SYN_PAGE;
+  const int chunk = (page_hi - page_lo + n_splits) / n_splits;
+  const int p0 = page_lo + split * chunk, p1 = min(p0 + chunk, page_hi + 1);
+  const int n_qs = R / KS, n_dt = rank / 16;
+
+  frag qf[QS];
+  const bf16* qrow = q + ((size_t)(start + tok) * nh + head) * R + g * PIECE;
+#pragma unroll
+  for (int ks = 0; ks < QS; ++ks)
+    if (ks < n_qs) qf[ks] = *(const frag*)(qrow + ks * KS);
+
+  f32x4 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int* pages = page_table + (size_t)seq * table_stride;
+  for (int p = p0; p < p1; ++p) {
+    const int page = pages[p];
+    const bf16* kb = k_pages + (size_t)page * SYN_PAGE * R + (size_t)i * R + g * PIECE;
+    f32x4 s[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < QS; ++ks)
+      if (ks < n_qs) {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+          const frag a = *(const frag*)(kb + (size_t)kt * 16 * R + ks * KS);
+          s[kt] = la_mfma(a, qf[ks], s[kt]);
+        }
+      }
+    // s[kt][e]: key p * 64 + kt * 16 + 4 g + e against this lane's row
+    const int key0 = p * SYN_PAGE + 4 * g;
+    float top = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + kt * 16 + e;
+        const bool seen = key <= pos && (window <= 0 || pos - key < window);
+        s[kt][e] = seen ? s[kt][e] * scale : -INFINITY;
+        top = fmaxf(top, s[kt][e]);
+      }
+    top = fmaxf(top, __shfl_xor(top, 16, SYN_WAVE));
+    top = fmaxf(top, __shfl_xor(top, 32, SYN_WAVE));
+    const float m_new = fmaxf(m, top);
+    const float base = m_new == -INFINITY ? 0.f : m_new;          // (a row that sees nothing of this page)
+    const float alpha = expf(m - base);
+    float sum = 0.f;
+    bf16x4 hi[4], lo[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = expf(s[kt][e] - base);
+        sum += w;
+        hi[kt][e] = (bf16)w;
+        lo[kt][e] = (bf16)(w - (float)hi[kt][e]);
+      }
+    sum += __shfl_xor(sum, 16, SYN_WAVE);
+    sum += __shfl_xor(sum, 32, SYN_WAVE);
+    l = l * alpha + sum;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      if (dt < n_dt) acc[dt] *= alpha;
+    // slots behind the sequence's end may hold anything: their weights are 0, their values are made 0 as well
+    const int left = kv_len - p * SYN_PAGE;
+    const bf16* vb = v_pages + (size_t)page * rank * SYN_PAGE + (size_t)i * SYN_PAGE + 4 * g;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      bf16x8 ph, pl;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ph[e] = hi[2 * half][e], ph[4 + e] = hi[2 * half + 1][e];
+        pl[e] = lo[2 * half][e], pl[4 + e] = lo[2 * half + 1][e];
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        if (dt < n_dt) {
+          const bf16* vr = vb + (size_t)dt * 16 * SYN_PAGE + 32 * half;
+          const bf16x4 v0 = *(const bf16x4*)vr, v1 = *(const bf16x4*)(vr + 16);
+          bf16x8 a;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[e] = v0[e], a[4 + e] = v1[e];
+          if (left < SYN_PAGE) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (32 * half + 4 * g + e >= left) a[e] = (bf16)0.f;
+              if (32 * half + 16 + 4 * g + e >= left) a[4 + e] = (bf16)0.f;
+            }
+          }
+          acc[dt] = la_mfma(a, ph, acc[dt]);
+          acc[dt] = la_mfma(a, pl, acc[dt]);
+        }
+    }
+  }
+  // acc[dt][e]: value dt * 16 + 4 g + e of this lane's row
+  if (n_splits == 1) {
+    if (!row_ok) return;
+    const float inv = 1.f / l;
+    bf16* orow = out + ((size_t)(start + tok) * nh + head) * rank + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      if (dt < n_dt) {
+        bf16x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = (bf16)(acc[dt][e] * inv);
+        *(bf16x4*)(orow + dt * 16) = r;
+      }
+  } else {
+    const size_t at = ((size_t)gt * n_splits + split) * LA_ROWS + i;
+    if (g == 0) part_ml[2 * at] = m, part_ml[2 * at + 1] = l;
+    float* prow = part_o + at * rank + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      if (dt < n_dt) *(f32x4*)(prow + dt * 16) = acc[dt];
+  }
+}
+
+// the splits of a tile merged in their order: the largest maximum, every split's sum and values scaled to it
+__global__ void __launch_bounds__(256)
+latent_attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                              const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int nh, int rank,
+                              int n_splits) {
+  const int gt = blockIdx.x;
+  int seq, tile, start, rows;
+  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;
+  for (int r = 0; r < LA_ROWS; ++r) {
+    const int flat = tile * LA_ROWS + r;
+    if (flat >= rows) break;
+    const size_t at0 = (size_t)gt * n_splits * LA_ROWS + r;
+    float mm = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[2 * (at0 + (size_t)s * LA_ROWS)]);
+    float l = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float ms = part_ml[2 * (at0 + (size_t)s * LA_ROWS)];
+      l += (ms == -INFINITY ? 0.f : expf(ms - mm)) * part_ml[2 * (at0 + (size_t)s * LA_ROWS) + 1];
+    }
+    bf16* orow = out + ((size_t)(start + flat / nh) * nh + flat % nh) * rank;
+    for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+      float o = 0.f;
+      for (int s = 0; s < n_splits; ++s) {
+        const size_t at = at0 + (size_t)s * LA_ROWS;
+        const float ms = part_ml[2 * at];
+        if (ms != -INFINITY) o += expf(ms - mm) * part_o[at * rank + d];
+      }
+      orow[d] = (bf16)(o / l);
+    }
+  }
+}
+
+// n_tiles: at least the number of tiles of all sequences, sum_b ceil(new tokens_b * heads / 16) (the host may not know
+// the counts: (n_tokens * heads + 15) / 16 + n_seqs bounds it).  workspace: floats for n_tiles * n_splits * 16 *
+// (rank + 2), used when n_splits > 1.
+SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                         int table_stride, const int* seq_start, const int* seq_past, int n_seqs,
+                                         void* out, float* workspace, long workspace_floats, float scale, int n_tiles,
+                                         int nh, int rank, int rot, int window, int n_splits, hipStream_t stream) {
+  const int R = rank + rot;
+  SYN_CHECK(n_seqs > 0 && n_tiles > 0 && nh > 0, "latent_attention: empty input");
+  SYN_CHECK(rank > 0 && rank % 16 == 0 && rank <= 512 && R % 16 == 0 && R <= 640,
+            "latent_attention: rows of %d + %d values (multiples of 16 up to 512 and 640 together)", rank, rot);
+  SYN_CHECK(window >= 0 && n_splits >= 1, "latent_attention: window %d, %d splits", window, n_splits);
+  SYN_CHECK(n_splits == 1 || (workspace != nullptr && workspace_floats >= (long)n_tiles * n_splits * LA_ROWS * (rank + 2)),
+            "latent_attention: a workspace of %ld floats for %d tiles in %d splits", workspace_floats, n_tiles, n_splits);
+  float* part_o = workspace;
+  float* part_ml = workspace ? workspace + (size_t)n_tiles * n_splits * LA_ROWS * rank : nullptr;
+  const dim3 grid((n_tiles + 3) / 4, n_splits);
+  const bool x32 = R % 32 == 0;
+#define SYN_LA(DT, QS, X)                                                                                             \
+  latent_attention_bf16_kernel<DT, QS, X><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,              \
+      (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs, (bf16*)out, part_o, part_ml, scale,  \
+      nh, rank, R, window, n_splits)
+  if (rank <= 128 && R <= 160) {
+    if (x32) SYN_LA(8, 5, true); else SYN_LA(8, 10, false);
+  } else if (rank <= 256 && R <= 320) {
+    if (x32) SYN_LA(16, 10, true); else SYN_LA(16, 20, false);
+  } else {
+    if (x32) SYN_LA(32, 20, true); else SYN_LA(32, 40, false);
+  }
+#undef SYN_LA
+  SYN_LAUNCH_CHECK("latent_attention");
+  if (n_splits > 1) {
+    latent_attention_merge_kernel<<<(n_tiles + 3) / 4 * 4, 256, 0, stream>>>(part_o, part_ml, seq_start, n_seqs,
+                                                                             (bf16*)out, nh, rank, n_splits);
+    SYN_LAUNCH_CHECK("latent_attention_merge");
+  }
+  return 0;
+}

@@ -1223,18 +1223,70 @@ def latent_intake(proj, gain, eps, cos, sin, q_nope, q_full, k_pages, v_pages, p
 
 # ----------------------------------------------------------------------------- latent attention
 
-LATENT_ATTENTION_MAX_ROW = WINDOW_ATTENTION_MAX_DIM
+LATENT_ATTENTION_MAX_ROW = WINDOW_ATTENTION_MAX_DIM      # plain FMA: 32-bit, and sizes that the tiles do not take
+LATENT_TILED_MAX_RANK, LATENT_TILED_MAX_ROW = 512, 640
 
 
-def latent_attention_takes(rank, rot_dim) -> bool:
+def latent_attention_tiled(rank, rot_dim) -> bool:
+    """Whether the bf16 kernel on the matrix cores takes these sizes."""
+    return (rank % 16 == 0 and (rank + rot_dim) % 16 == 0 and 0 < rank <= LATENT_TILED_MAX_RANK
+            and rank + rot_dim <= LATENT_TILED_MAX_ROW)
+
+
+def latent_attention_takes(rank, rot_dim, dtype=_F32) -> bool:
+    if dtype == _BF16 and latent_attention_tiled(rank, rot_dim):
+        return True
     return 0 < rank and rank + rot_dim <= LATENT_ATTENTION_MAX_ROW
 
 
-def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, rank, rot_dim, window=0):
+def _latent_tiles(n_tokens, n_heads, n_seqs, max_pages):
+    """(a bound on the tiles of 16 (token, head) rows, the splits of a tile's pages): many tiles run whole, few are cut
+    until some 2,048 waves have work."""
+    tiles = (n_tokens * n_heads + 15) // 16 + n_seqs
+    return tiles, max(1, min(int(max_pages), 2048 // tiles))
+
+
+def latent_attention_workspace(n_tokens, n_heads, n_seqs, rank, max_pages) -> int:
+    """Floats of workspace that latent_attention needs for a step of these sizes (0: none)."""
+    tiles, splits = _latent_tiles(n_tokens, n_heads, n_seqs, max_pages)
+    return tiles * splits * 16 * (rank + 2) if splits > 1 else 0
+
+
+def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, rank, rot_dim, window=0,
+                     seqs=None, workspace=None, force_simt=False):
     """Attention of `n_heads` queries a token over one shared key row a cached token: q_full [N, heads * (rank +
     rot_dim)], key rows k_pages [pages, 1, 64, rank + rot_dim] whose first `rank` values are the row's value (v_pages
     [pages, 1, rank, 64] holds them once more, along the keys); out [N, heads * rank] = sum_j softmax_j(scale q . k_j)
     k_j[:rank] over the keys at or before the query's position (window > 0: the last `window` of them).  Scores,
-    weights and sums are 32-bit."""
-    window_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, 1, rank + rot_dim,
-                     rank, window=window)
+    weights and sums are 32-bit.  seqs = (seq_start [B + 1], seq_past [B]): the step's sequences, whose new tokens lie
+    one after another at positions seq_past[b] ..; with them bf16 runs in tiles on the matrix cores where the sizes
+    allow (latent_attention_tiled), with `workspace` floats (latent_attention_workspace) for tiles cut into splits."""
+    R = rank + rot_dim
+    if q_full.dtype == _BF16 and seqs is not None and latent_attention_tiled(rank, rot_dim) and not force_simt:
+        seq_start, seq_past = seqs
+        _need(q_full, "latent_attention.q", _BF16, (None, n_heads * R))
+        N = q_full.shape[0]
+        _need(k_pages, "latent_attention.k_pages", _BF16, (None, 1, PAGE_TOKENS, R))
+        _need(v_pages, "latent_attention.v_pages", _BF16, (k_pages.shape[0], 1, rank, PAGE_TOKENS))
+        _need(page_table, "latent_attention.page_table", _I32, (None, None))
+        _need(seq_past, "latent_attention.seq_past", _I32, (None,))
+        B = seq_past.shape[0]
+        _need(seq_start, "latent_attention.seq_start", _I32, (B + 1,))
+        if page_table.shape[0] < B:
+            raise KernelError(f"latent_attention: page table has {page_table.shape[0]} rows for {B} sequences")
+        _need(out, "latent_attention.out", _BF16, (N, n_heads * rank))
+        tiles, splits = _latent_tiles(N, n_heads, B, page_table.shape[1])
+        floats = 0
+        if splits > 1:
+            need = tiles * splits * 16 * (rank + 2)
+            if workspace is None:
+                workspace = torch.empty(need, dtype=_F32, device=q_full.device)
+            _need(workspace, "latent_attention.workspace", _F32, (None,))
+            floats = workspace.shape[0]
+            if floats < need:
+                raise KernelError(f"latent_attention: a workspace of {floats} floats, {need} needed")
+        _call(load_library("core"), "syn_latent_attention_bf16", _ptr(q_full), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+              page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, _ptr(out), _ptr(workspace if splits > 1 else None),
+              ctypes.c_long(floats), ctypes.c_float(scale), tiles, n_heads, rank, rot_dim, int(window or 0), splits, _stream())
+        return
+    window_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, 1, R, rank, window=window)

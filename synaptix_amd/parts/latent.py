@@ -86,9 +86,10 @@ class LatentAttention(Mixer):
         return KvNeed(1, self.rank + self.rot, self.window, v_dim=self.rank)
 
     def check(self, dtype):
-        if not ops.latent_attention_takes(self.rank, self.rot):
-            raise ValueError(f"{self.prefix}: a cache row of {self.rank} + {self.rot} values "
-                             f"(at most {ops.LATENT_ATTENTION_MAX_ROW})")
+        if not ops.latent_attention_takes(self.rank, self.rot, dtype):
+            raise ValueError(f"{self.prefix}: a cache row of {self.rank} + {self.rot} values (at most "
+                             f"{ops.LATENT_ATTENTION_MAX_ROW}; in bfloat16 multiples of 16 up to {ops.LATENT_TILED_MAX_RANK} "
+                             f"and {ops.LATENT_TILED_MAX_ROW} together)")
         cos, _ = self.position.tables("cpu")
         if cos is not None and 2 * cos.shape[1] > self.rot:
             raise ValueError(f"{self.prefix}: the rotation turns {2 * cos.shape[1]} values, the rotated part has {self.rot}")
@@ -107,8 +108,10 @@ class LatentAttention(Mixer):
         # the query in the latent's space, into the first `rank` places of each head's row
         ops.heads_product(q_nope.view(N, nh, dim), self.w_uk_t, q_full.view(N, nh, R))
         o_lat = torch.empty((N, nh * rank), dtype=act, device=dev)
-        ops.latent_attention(q_full, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o_lat, self.scale, nh, rank, rot,
-                             window=self.window or 0)
+        floats = ops.latent_attention_workspace(N, nh, ctx.n_seqs, rank, table.shape[1]) if act == torch.bfloat16 else 0
+        ops.latent_attention(q_full, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o_lat, self.scale, nh,
+                             rank, rot, window=self.window or 0, seqs=(ctx.seq_start, ctx.seq_past),
+                             workspace=ctx.scratch("latent_attention", floats) if floats else None)
         o = torch.empty((N, nh * vdim), dtype=act, device=dev)
         gate = proj[:, nh * (dim + rot) + R:] if self.gate else None
         ops.heads_product(o_lat.view(N, nh, rank), self.w_uv, o.view(N, nh, vdim), gate=gate,

@@ -184,6 +184,64 @@ def test_latent_attention_sees_exactly_its_keys(window, dtype):
         assert float((one.cpu().double().view(H, C) - want[t]).abs().max()) < tol, f"query {t} alone"
 
 
+@pytest.mark.parametrize("H,C,B", [(3, 16, 16), (16, 32, 16), (5, 48, 0), (2, 144, 48), (20, 256, 64), (4, 512, 64)])
+@pytest.mark.parametrize("window", [0, 1, 64, 65, 130])
+def test_latent_attention_in_tiles_on_the_matrix_cores(window, H, C, B):
+    """The bf16 kernel whose tiles are 16 (token, head) rows of one sequence, for every size of its register tiles, with
+    k-steps of 16 and of 32: two sequences in one step, the second continuing from 70 cached rows (a portion that
+    starts inside a page); then single tokens of both sequences together, whose pages are cut into splits and merged.
+    Rows and queries as in the test above (a wrong or lost key shows); slots behind a sequence's end hold NaN."""
+    from synaptix_amd.kernels import ops
+    R, dt = C + B, torch.bfloat16
+    lens, past = [150, 210], [0, 70]
+    g = torch.Generator().manual_seed(window + H)
+    qs, rowss, wants = [], [], []
+    for T in lens:
+        kind = torch.randint(0, 3, (T,), generator=g)
+        kind[2] = 3
+        rows = 0.05 * torch.randn(T, R, generator=g, dtype=P.F64)
+        rows[torch.arange(T), C - 4 + kind] += 1.0
+        rows[:, :C - 4] += torch.randn(T, C - 4, generator=g, dtype=P.F64)
+        q = torch.zeros(T, H, R, dtype=P.F64)
+        q[torch.arange(T), :, C - 4 + kind] = 8.0
+        for t in (T - 1, T - 30, 100):
+            q[t] = 0
+            q[t, :, C - 1] = 12.0
+        q, rows = rounded(dt, q, rows)
+        qs.append(q), rowss.append(rows), wants.append(P.shared_row_attention(q, rows, C, 1.25, window or None))
+    # the two sequences' pages side by side in one pool; what lies behind a sequence's end is NaN
+    pools = [paged_rows(r, C, torch.float32, shuffle_seed=5 + j) for j, r in enumerate(rowss)]
+    n0 = pools[0][0].shape[0]
+    kp = torch.cat([pools[0][0], pools[1][0]]).float()
+    vp = torch.cat([pools[0][1], pools[1][1]]).float()
+    width = max(p[2].shape[1] for p in pools)
+    table = torch.zeros((2, width), dtype=torch.int32, device=DEV)
+    for j, (_, _, tb) in enumerate(pools):
+        table[j, :tb.shape[1]] = tb[0] + (n0 if j else 0)
+        last, used = int(table[j, (lens[j] - 1) // 64]), (lens[j] - 1) % 64 + 1
+        kp[last, 0, used:] = float("nan")
+        vp[last, 0, :, used:] = float("nan")
+    kp, vp = kp.to(dt), vp.to(dt)
+    new = [lens[0] - past[0], lens[1] - past[1]]
+    q_step = torch.cat([qs[0][past[0]:], qs[1][past[1]:]]).reshape(-1, H * R)
+    want = torch.cat([wants[0][past[0]:], wants[1][past[1]:]])
+    seqs = (torch.tensor([0, new[0], new[0] + new[1]], dtype=torch.int32, device=DEV),
+            torch.tensor(past, dtype=torch.int32, device=DEV))
+    out = torch.empty((q_step.shape[0], H * C), dtype=dt, device=DEV)
+    ops.latent_attention(dev(q_step, dt), kp, vp, table, None, None, out, 1.25, H, C, B, window=window, seqs=seqs)
+    assert float((out.cpu().double().view(-1, H, C) - want).abs().max()) < 2e-2
+    # the last tokens alone, one of each sequence: their pages in splits
+    for back in (1, 30):
+        q1 = torch.stack([qs[0][lens[0] - back], qs[1][lens[1] - back]]).reshape(2, H * R)
+        seqs1 = (torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
+                 torch.tensor([lens[0] - back, lens[1] - back], dtype=torch.int32, device=DEV))
+        assert ops.latent_attention_workspace(2, H, 2, C, width) > 0
+        one = torch.empty((2, H * C), dtype=dt, device=DEV)
+        ops.latent_attention(dev(q1, dt), kp, vp, table, None, None, one, 1.25, H, C, B, window=window, seqs=seqs1)
+        w1 = torch.stack([wants[0][lens[0] - back], wants[1][lens[1] - back]])
+        assert float((one.cpu().double().view(2, H, C) - w1).abs().max()) < 2e-2, f"single tokens {back} from the end"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,D,B,C,pairs", [(3, 8, 6, 20, 3), (2, 16, 8, 32, 2), (1, 4, 0, 6, 0), (4, 32, 16, 64, 8)])
 def test_latent_intake_norms_turns_and_writes_the_pages(H, D, B, C, pairs, dtype):
