@@ -2,7 +2,7 @@
 """Throughput of the engine at a Qwen3 shape with random bf16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|4b|32b] [--batch 8] [--layers L]
-    python bench.py --design bizipel [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
+    python bench.py --design bizipel|kamivik [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
 
 --shape 8b (the default) and 32b: a step is one decode step of `batch` sequences, each after a
 2,048-token prompt of uniform ids, run through the same captured graph and host loop that
@@ -25,6 +25,9 @@ own clock over its last `steps` decode steps, to stand beside `value`), the 4b w
 --design bizipel: another run than the default one.  Prefill and decode throughput of the Bizipel design at a few layer sizes
 beside the Qwen3 decoder at the same sizes (width, heads, head size, feed-forward, vocabulary, layers; random bf16
 weights), each with the time of every kernel entry point of one prompt step and one decode step; one JSON line.
+--design kamivik: the same for the Kamivik design: latent attention with a latent of 512 and a rotated part of 64 beside
+unrotated keys and values of the head size, every second layer with the window; a mixture of 8 x top experts of which each
+token uses `top`, top x the expert's width being the dense feed-forward's width.
 
 Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
 crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
@@ -174,16 +177,34 @@ SIDE_BY_SIDE_SIZES = {     # layers, width, heads, kv heads, head size, feed-for
 }
 
 
-def design_configs(size, window, context):
-    """(Qwen3 configuration, Bizipel configuration) of one size: the same width, attention heads, feed-forward,
-    vocabulary (tied) and number of layers; the Bizipel layers add a matrix memory of heads / 4 heads (keys of 64,
-    values of 128), two residual streams and a window that keeps 4 first keys."""
+KAMIVIK_EXPERTS = {"small": (4, 1024), "mid": (4, 2048), "large": (6, 2048)}      # (top, an expert's width); 8 x top experts
+
+
+def design_configs(design, size, window, context):
+    """(Qwen3 configuration, the other design's configuration) of one size: the same width, attention heads,
+    feed-forward, vocabulary and number of layers.  The Bizipel layers add a matrix memory of heads / 4 heads (keys of
+    64, values of 128), two residual streams and a window that keeps 4 first keys (vocabulary tied).  The Kamivik
+    layers have latent attention (a latent of 512, 64 rotated values, unrotated keys and values of the head size; every
+    second layer with the window) and a mixture of experts whose active width equals the dense feed-forward's."""
     from synaptix_amd import Qwen3Config
-    from synaptix_amd.config import BizipelConfig
+    from synaptix_amd.config import BizipelConfig, KamivikConfig
     L, W, nh, nkv, hd, ff, V = SIDE_BY_SIDE_SIZES[size]
     qwen = Qwen3Config.from_dict(dict(_COMMON, num_hidden_layers=L, hidden_size=W, num_attention_heads=nh,
                                       num_key_value_heads=nkv, head_dim=hd, intermediate_size=ff, vocab_size=V,
-                                      tie_word_embeddings=True, max_position_embeddings=context))
+                                      tie_word_embeddings=design == "bizipel", max_position_embeddings=context))
+    if design == "kamivik":
+        top, eff = KAMIVIK_EXPERTS[size]
+        layers = []
+        for i in range(L):
+            mixer = {"heads": nh, "dim": hd, "rot_dim": 64, "vdim": hd, "kv_rank": 512, "scale": (hd + 64) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": 64}}
+            if i % 2:
+                mixer["mask"] = {"size": window}
+            layers.append({"type": "latent_attention_2" if i % 2 else "latent_attention", "mixer": mixer,
+                           "mlp": {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": 8 * top, "top": top}}})
+        kam = KamivikConfig.from_dict({"architecture": "Kamivik", "vocab": V, "width": W, "norm": {"eps": 1e-6},
+                                       "residual_mult": 0.5, "layers": layers})
+        return qwen, kam
     layer = {"type": "parallel",
              "mixer": {"left": {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
                                 "mask": {"size": window, "keep_first": 4}},
@@ -209,11 +230,18 @@ def designs_side_by_side(args) -> int:
     context = P + steps + warmup + 72
     points = {}
     for size in sizes:
-        for design, cfg in zip(("qwen3", "bizipel"), design_configs(size, args.window, context)):
+        for design, cfg in zip(("qwen3", args.design), design_configs(args.design, size, args.window, context)):
             torch.manual_seed(0)
             eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=(B + 1) * ((context + 63) // 64 * 64),
                                      max_seq=context if design == "qwen3" else None)
             weight_bytes = sum(2 * int(torch.Size(sp.shape).numel()) for sp in eng.model.tensor_specs().values())
+            if design == "kamivik":
+                # a decode step reads the experts that its tokens chose, not all of them: the expected number of
+                # distinct ones among B x top uniform choices of 8 x top
+                top, eff = KAMIVIK_EXPERTS[size]
+                E, one = 8 * top, 2 * 2 * eff * cfg.width
+                touched = E * (1.0 - (1.0 - top / E) ** B)
+                weight_bytes -= int(len(cfg.layers) * (E - touched) * one)
             g = torch.Generator().manual_seed(0)
             prompt = torch.randint(0, cfg.vocab_size, (P,), generator=g).tolist()
             times = []
@@ -255,12 +283,13 @@ def designs_side_by_side(args) -> int:
             gc.collect()
             torch.cuda.empty_cache()
     first = sizes[0]
-    line = {"metric": f"decode tok/s at batch {B} of the Bizipel design at the {first} size (the Qwen3 decoder at equal sizes "
-                      f"and prefill at {P} tokens in points), bf16", "value": points[f"{first}_bizipel_decode_b{B}_tok_s"],
+    name = args.design.capitalize()
+    line = {"metric": f"decode tok/s at batch {B} of the {name} design at the {first} size (the Qwen3 decoder at equal sizes "
+                      f"and prefill at {P} tokens in points), bf16", "value": points[f"{first}_{args.design}_decode_b{B}_tok_s"],
             "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
-            "ms_per_step": points[f"{first}_bizipel_decode_b{B}_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "ms_per_step": points[f"{first}_{args.design}_decode_b{B}_ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
-            "config": {"model": "Bizipel beside Qwen3 at equal layer sizes", "sizes": {s: list(SIDE_BY_SIDE_SIZES[s]) for s in sizes},
+            "config": {"model": f"{name} beside Qwen3 at equal layer sizes", "sizes": {s: list(SIDE_BY_SIDE_SIZES[s]) for s in sizes},
                        "global_batch": B, "seq_len": P, "window": args.window, "parallelism": "single GPU",
                        "graph": not args.no_graph},
             "points": points}
@@ -283,7 +312,7 @@ def main() -> int:
                     help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", default=None, choices=["bizipel"],
+    ap.add_argument("--design", default=None, choices=["bizipel", "kamivik"],
                     help="another run than the default one: this design beside the Qwen3 decoder at equal layer sizes")
     ap.add_argument("--sizes", default="small,mid,large", help="with --design: which of small, mid, large")
     ap.add_argument("--window", type=int, default=1024, help="with --design: the keys a query of the new design sees")

@@ -9,11 +9,12 @@
 //     number of elements from one group to the next.
 // Epilogue, in this order and each optional: the exact GELU 0.5 z (1 + erf(z / sqrt 2)); a weight of the row;
 // sigmoid of a gate value read from float rows.  Sums are 32-bit.  bf16 operands whose K is a multiple of 32 run on
-// the matrix cores (16x16x32, operands straight from memory as 16-byte pieces of rows, no LDS: a wave computes 32
-// rows x 64 columns); everything else, and all of the 32-bit path, is plain FMA with one wave a (row, 8 columns).
+// the matrix cores: with few rows a group 16x16x32 with operands straight from memory as 16-byte pieces of rows (no
+// LDS: a wave computes 32 rows x 64 columns), with many rows tiles of 128 x 128 through LDS (any K that is a multiple
+// of 8); everything else, and all of the 32-bit path, is plain FMA with one wave a (row, 8 columns).
 //
-// Beside it: the router of a mixture of experts (logits, the largest `top` of them, softmax over those) and the
-// counting sort that turns its choices into segments.
+// Beside it: the choice of a mixture's router (the largest `top` logits of a token, softmax over those) and the
+// counting sort that turns the choices into segments.
 #include "common.h"
 
 struct GroupedArgs {
@@ -165,6 +166,119 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
   }
 }
 
+// ---------------------------------------------------------------- bf16 on the matrix cores, many rows a group
+// Tiles of 128 rows x 128 outputs x 32 k through LDS (double-buffered: while one k-tile is multiplied the next is on
+// its way from memory into registers), four waves of 64 x 64 each, MFMA 32x32x16: A = rows of x, B = rows of W,
+// D[m = 8 (e / 4) + 4 (lane / 32) + e % 4][n = lane % 32].  Rows of x are gathered through a_rows on their way into
+// LDS.  K is a multiple of 8 (a 16-byte chunk lies inside or outside as a whole).
+#define GT_BM 128
+#define GT_BN 128
+#define GT_BK 32
+#define GT_LD (GT_BK + 8)
+__global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs g) {
+  __shared__ __attribute__((aligned(16))) bf16 smem[2 * (GT_BM + GT_BN) * GT_LD];
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  int b = blockIdx.z, row0, row_end;
+  if (g.seg_start) {
+    int t = blockIdx.x;
+    b = -1;
+    for (int e = 0; e < g.groups; ++e) {
+      const int s0 = g.seg_start[e], n = g.seg_start[e + 1] - s0, tiles = (n + GT_BM - 1) / GT_BM;
+      if (t < tiles) {
+        b = e, row0 = s0 + t * GT_BM, row_end = s0 + n;
+        break;
+      }
+      t -= tiles;
+    }
+    if (b < 0) return;                      // (the whole workgroup, before any barrier)
+  } else {
+    row0 = blockIdx.x * GT_BM, row_end = g.M;
+    if (row0 >= row_end) return;
+  }
+  const int n0 = blockIdx.y * GT_BN;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+  constexpr int CPR = GT_BK / 8, RPP = 256 / CPR, XL = GT_BM / RPP, WL = GT_BN / RPP;
+  const int lrow = tid / CPR, lchunk = (tid % CPR) * 8;
+  const bf16* A = (const bf16*)g.a + (size_t)b * g.a_group;
+  const bf16* W = (const bf16*)g.w + (size_t)b * g.w_group;
+  const bf16* xg[XL];
+  const bf16* wg[WL];
+  bool xin[XL], win[WL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int r = row0 + lrow + RPP * i;
+    xin[i] = r < row_end;
+    const int src = xin[i] ? (g.a_rows ? g.a_rows[r] : r) : 0;
+    xg[i] = A + (size_t)src * g.lda + lchunk;
+  }
+#pragma unroll
+  for (int i = 0; i < WL; ++i) {
+    const int n = n0 + lrow + RPP * i;
+    win[i] = n < g.N;
+    wg[i] = W + (size_t)(win[i] ? n : 0) * g.ldw + lchunk;
+  }
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int nk = (g.K + GT_BK - 1) / GT_BK;
+  bf16x8 rx[XL], rw[WL];
+  auto fetch = [&](int kt) {
+    const int k = kt * GT_BK;
+    const bool kin = k + lchunk < g.K;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) rx[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + k) : zero;
+#pragma unroll
+    for (int i = 0; i < WL; ++i) rw[i] = (kin && win[i]) ? *(const bf16x8*)(wg[i] + k) : zero;
+  };
+  auto stash = [&](int buf) {
+    bf16* xs = smem + buf * (GT_BM + GT_BN) * GT_LD;
+    bf16* ws = xs + GT_BM * GT_LD;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs + (lrow + RPP * i) * GT_LD + lchunk) = rx[i];
+#pragma unroll
+    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws + (lrow + RPP * i) * GT_LD + lchunk) = rw[i];
+  };
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int fr = lane % 32, fk = (lane / 32) * 8;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) fetch(kt + 1);
+    const bf16* xs = smem + buf * (GT_BM + GT_BN) * GT_LD;
+    const bf16* ws = xs + GT_BM * GT_LD;
+#pragma unroll
+    for (int ks = 0; ks < GT_BK; ks += 16) {
+      bf16x8 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = *(const bf16x8*)(xs + (wm + i * 32 + fr) * GT_LD + ks + fk);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = *(const bf16x8*)(ws + (wn + j * 32 + fr) * GT_LD + ks + fk);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) stash(buf ^ 1);      // the other buffer was last read before the previous barrier
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = row0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const int n = n0 + wn + j * 32 + lane % 32;
+        if (r < row_end && n < g.N) grouped_store(g, r, b, n, grouped_epilogue(g, acc[i][j][e], r, b, n));
+      }
+}
+
 // rows_bound: with segments, the number of rows in all segments together (what the index lists hold)
 SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const void* w, long w_group, long ldw, void* out,
                                    long ldo, long o_group, int in_is_f32, int out_is_f32, const int* seg_start,
@@ -181,7 +295,15 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
                          row_weight, gate, gate_ld, gate_group, gate_col, act, M, N, K, groups};
   const bool aligned = K % 32 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ldw % 8 == 0 && w_group % 8 == 0 &&
                        (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
-  if (!in_is_f32 && aligned && !force_simt) {
+  // many rows a group (on average, where the host does not know the segments): the tiles through LDS
+  const long rows_a_group = seg_start ? rows_bound / groups : M;
+  const bool chunks = K % 8 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ldw % 8 == 0 && w_group % 8 == 0 &&
+                      (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+  if (!in_is_f32 && chunks && force_simt == 0 && rows_a_group >= 48) {
+    const int row_tiles = seg_start ? (rows_bound + GT_BM - 1) / GT_BM + groups : (M + GT_BM - 1) / GT_BM;
+    const dim3 grid(row_tiles, (N + GT_BN - 1) / GT_BN, seg_start ? 1 : groups);
+    grouped_product_tiled_kernel<<<grid, 256, 0, stream>>>(g);
+  } else if (!in_is_f32 && aligned && force_simt != 1) {
     const int row_tiles = seg_start ? (rows_bound + GP_TM - 1) / GP_TM + groups : (M + GP_TM - 1) / GP_TM;
     const dim3 grid(row_tiles, (N + 255) / 256, seg_start ? 1 : groups);
     grouped_product_mfma_kernel<<<grid, 256, 0, stream>>>(g);
@@ -194,27 +316,24 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
   return 0;
 }
 
-// ---------------------------------------------------------------- router: logits, the largest `top`, their softmax
-// One workgroup a token.  z[e] = sum_k x[k] W[e, k] + bias[e] in 32-bit; of equal logits the lower index comes first.
+// ---------------------------------------------------------------- router: the largest `top` logits, their softmax
+// One wave a token over its row of logits z [E] (32-bit sums of a product that ran before) + bias; of equal logits
+// the lower index comes first.
 #define ROUTE_MAX_EXPERTS 1024
 #define ROUTE_MAX_TOP 64
-template <typename T>
-__global__ void __launch_bounds__(256) route_topk_kernel(const T* __restrict__ x, const T* __restrict__ w,
-                                                         const float* __restrict__ bias, int* __restrict__ ids,
-                                                         float* __restrict__ weights, int H, int E, int top) {
-  __shared__ float z[ROUTE_MAX_EXPERTS];
-  __shared__ float chosen[ROUTE_MAX_TOP];
-  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, tok = blockIdx.x;
-  const T* xr = x + (size_t)tok * H;
-  for (int e = wave; e < E; e += 4) {
-    const T* wr = w + (size_t)e * H;
-    float acc = 0.f;
-    for (int k = lane; k < H; k += SYN_WAVE) acc = fmaf(to_f32<T>(xr[k]), to_f32<T>(wr[k]), acc);
-    acc = wave_sum(acc);
-    if (lane == 0) z[e] = acc + (bias ? bias[e] : 0.f);
-  }
-  __syncthreads();
-  if (wave != 0) return;
+__global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                         int* __restrict__ ids, float* __restrict__ weights,
+                                                         int n_tokens, int E, int top) {
+  __shared__ float zs[4][ROUTE_MAX_EXPERTS];
+  __shared__ float chosen_s[4][ROUTE_MAX_TOP];
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, tok = blockIdx.x * 4 + wave;
+  if (tok >= n_tokens) return;             // (waves work alone: no barrier of the workgroup below)
+  float* z = zs[wave];
+  float* chosen = chosen_s[wave];
+  for (int e = lane; e < E; e += SYN_WAVE) z[e] = logits[(size_t)tok * E + e] + (bias ? bias[e] : 0.f);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   for (int t = 0; t < top; ++t) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -246,15 +365,12 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const T* __restrict__ x
   }
 }
 
-SYN_EXPORT int syn_route_topk(const void* x, const void* w, int is_f32, const float* bias, int* ids, float* weights,
-                              int n_tokens, int H, int E, int top, hipStream_t stream) {
-  SYN_CHECK(n_tokens > 0 && H > 0, "route_topk: empty input");
+SYN_EXPORT int syn_route_topk(const float* logits, const float* bias, int* ids, float* weights, int n_tokens, int E,
+                              int top, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0, "route_topk: empty input");
   SYN_CHECK(E > 0 && E <= ROUTE_MAX_EXPERTS, "route_topk: %d experts (at most %d)", E, ROUTE_MAX_EXPERTS);
   SYN_CHECK(top > 0 && top <= E && top <= ROUTE_MAX_TOP, "route_topk: the %d largest of %d (at most %d)", top, E, ROUTE_MAX_TOP);
-  if (is_f32)
-    route_topk_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)x, (const float*)w, bias, ids, weights, H, E, top);
-  else
-    route_topk_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, bias, ids, weights, H, E, top);
+  route_topk_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, bias, ids, weights, n_tokens, E, top);
   SYN_LAUNCH_CHECK("route_topk");
   return 0;
 }

@@ -2,7 +2,9 @@
 //
 //   q       [N][heads][R]        R = rank + rot: the query in the latent's space, then its rotated part
 //   k_pages [pages][64][R]       a token's row [latent | rotated key part]
-//   v_pages [pages][rank][64]    the latent once more, along the keys
+//   v_pages [pages][rank x 64]   the latent once more, in the order of this kernel's fragments (la_v_offset): the
+//                                8 values that a lane feeds into one matrix instruction lie together, a wave's 64
+//                                lanes one after another: a fragment is 1 KB of consecutive bytes
 //   out     [N][heads][rank]     sum_j softmax_j(scale q . k_j) k_j[:rank]  over the keys j that the query sees:
 //                                j <= position, and position - j < window if there is a window
 //
@@ -15,8 +17,9 @@
 // order in which two score tiles leave them, and V^T's 8-byte pieces are fetched in that order too).  The scores
 // and weights are 32-bit; a weight meets V as two bf16 numbers (the weight rounded, and what the rounding left), so
 // it counts with 16 bits of mantissa although the product runs in bf16; sums are 32-bit.
-// A tile's pages may be cut into splits (grid y) whose partial results a second kernel merges: single tokens over
-// long sequences then fill the chip.
+// A tile's pages may be cut into splits (grid y) whose partial results a second kernel merges, and (SHARE) the four
+// waves of a workgroup may take one tile's pages in turns and merge through LDS: single tokens over long sequences
+// then fill the chip.
 #include "common.h"
 
 #define LA_ROWS 16
@@ -46,9 +49,17 @@ __device__ __forceinline__ bool la_find_tile(int t, const int* seq_start, int n_
   return false;
 }
 
+// Where value d of the token in slot `slot` of a page lies in a bf16 value page of latent attention: fragment (d / 16,
+// slot / 32), lane 16 g + d % 16, element e, with the 32 slots of a half in the order in which two tiles of scores
+// leave them in a lane: e < 4: slot 4 g + e; e >= 4: slot 16 + 4 g + (e - 4).
+__host__ __device__ __forceinline__ int la_v_offset(int d, int slot) {
+  const int half = slot >> 5, s = slot & 31, second = s >> 4, g = (s & 15) >> 2, e = (s & 3) + 4 * second;
+  return ((((d >> 4) * 2 + half) * 64 + g * 16 + (d & 15)) << 3) + e;
+}
+
 // DT: tiles of 16 values that the accumulators hold (rank <= 16 DT); QS: k-steps that the query's registers hold
 // (R <= QS * (X32 ? 32 : 16)); X32: k-steps of 32 (R a multiple of 32) or of 16.
-template <int DT, int QS, bool X32>
+template <int DT, int QS, bool X32, bool SHARE>
 __global__ void __launch_bounds__(256)
 latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                              const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
@@ -58,9 +69,10 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   typedef typename LaFrag<X32>::type frag;
   constexpr int KS = X32 ? 32 : 16, PIECE = KS / 4;
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, g = lane / 16;
-  const int gt = blockIdx.x * 4 + wave, split = blockIdx.y;
+  // SHARE: the workgroup's waves take one tile's pages in turns; else a tile a wave
+  const int gt = SHARE ? blockIdx.x : blockIdx.x * 4 + wave, split = blockIdx.y;
   int seq, tile, start, rows;
-  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;      // (no barrier anywhere below)
+  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;      // (SHARE: the whole workgroup)
   const int past = seq_past[seq];
   const int flat0 = tile * LA_ROWS, flat_last = min(flat0 + LA_ROWS, rows) - 1;
   const bool row_ok = flat0 + i < rows;
@@ -86,7 +98,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int* pages = page_table + (size_t)seq * table_stride;
-  for (int p = p0; p < p1; ++p) {
+  for (int p = SHARE ? p0 + wave : p0; p < p1; p += SHARE ? 4 : 1) {
     const int page = pages[p];
     const bf16* kb = k_pages + (size_t)page * SYN_PAGE * R + (size_t)i * R + g * PIECE;
     f32x4 s[4];
@@ -138,7 +150,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
       if (dt < n_dt) acc[dt] *= alpha;
     // slots behind the sequence's end may hold anything: their weights are 0, their values are made 0 as well
     const int left = kv_len - p * SYN_PAGE;
-    const bf16* vb = v_pages + (size_t)page * rank * SYN_PAGE + (size_t)i * SYN_PAGE + 4 * g;
+    const bf16* vb = v_pages + (size_t)page * rank * SYN_PAGE + lane * 8;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       bf16x8 ph, pl;
@@ -150,11 +162,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
         if (dt < n_dt) {
-          const bf16* vr = vb + (size_t)dt * 16 * SYN_PAGE + 32 * half;
-          const bf16x4 v0 = *(const bf16x4*)vr, v1 = *(const bf16x4*)(vr + 16);
-          bf16x8 a;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) a[e] = v0[e], a[4 + e] = v1[e];
+          bf16x8 a = *(const bf16x8*)(vb + (dt * 2 + half) * 512);
           if (left < SYN_PAGE) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -168,6 +176,35 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     }
   }
   // acc[dt][e]: value dt * 16 + 4 g + e of this lane's row
+  if constexpr (SHARE) {
+    // waves 1 .. 3 hand their maximum, sum and values to wave 0 through LDS, one after another
+    __shared__ float share_ml[2 * LA_ROWS];
+    __shared__ __attribute__((aligned(16))) float share_o[LA_ROWS * 16 * DT];
+    for (int w = 1; w < 4; ++w) {
+      if (wave == w) {
+        if (g == 0) share_ml[2 * i] = m, share_ml[2 * i + 1] = l;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          if (dt < n_dt) *(f32x4*)(share_o + (i * DT + dt) * 16 + 4 * g) = acc[dt];
+      }
+      __syncthreads();
+      if (wave == 0) {
+        const float mo = share_ml[2 * i], lo_ = share_ml[2 * i + 1];
+        const float mn = fmaxf(m, mo), base = mn == -INFINITY ? 0.f : mn;
+        const float fa = expf(m - base), fb = expf(mo - base);
+        l = l * fa + lo_ * fb;
+        m = mn;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          if (dt < n_dt) {
+            const f32x4 o = *(const f32x4*)(share_o + (i * DT + dt) * 16 + 4 * g);
+            acc[dt] = acc[dt] * fa + o * fb;
+          }
+      }
+      __syncthreads();
+    }
+    if (wave != 0) return;
+  }
   if (n_splits == 1) {
     if (!row_ok) return;
     const float inv = 1.f / l;
@@ -190,60 +227,68 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   }
 }
 
-// the splits of a tile merged in their order: the largest maximum, every split's sum and values scaled to it
+// the splits of a tile merged in their order: the largest maximum, every split's sum and values scaled to it.
+// One workgroup a (tile, row): the splits' factors once in LDS, then a thread a value.
+#define LA_MAX_SPLITS 1024
 __global__ void __launch_bounds__(256)
 latent_attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                               const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int nh, int rank,
                               int n_splits) {
-  const int gt = blockIdx.x;
+  __shared__ float factor[LA_MAX_SPLITS];
+  __shared__ float red[16];
+  const int gt = blockIdx.x, r = blockIdx.y;
   int seq, tile, start, rows;
   if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;
-  for (int r = 0; r < LA_ROWS; ++r) {
-    const int flat = tile * LA_ROWS + r;
-    if (flat >= rows) break;
-    const size_t at0 = (size_t)gt * n_splits * LA_ROWS + r;
-    float mm = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[2 * (at0 + (size_t)s * LA_ROWS)]);
-    float l = 0.f;
+  const int flat = tile * LA_ROWS + r;
+  if (flat >= rows) return;                 // (the whole workgroup)
+  const size_t at0 = (size_t)gt * n_splits * LA_ROWS + r;
+  float mm = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[2 * (at0 + (size_t)s * LA_ROWS)]);
+  float part = 0.f;
+  for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
+    const size_t at = at0 + (size_t)s * LA_ROWS;
+    const float ms = part_ml[2 * at];
+    const float f = ms == -INFINITY ? 0.f : expf(ms - mm);
+    factor[s] = f;
+    part += f * part_ml[2 * at + 1];
+  }
+  const float l = block_sum(part, red);     // (its barriers also publish `factor`)
+  bf16* orow = out + ((size_t)(start + flat / nh) * nh + flat % nh) * rank;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float o = 0.f;
     for (int s = 0; s < n_splits; ++s) {
-      const float ms = part_ml[2 * (at0 + (size_t)s * LA_ROWS)];
-      l += (ms == -INFINITY ? 0.f : expf(ms - mm)) * part_ml[2 * (at0 + (size_t)s * LA_ROWS) + 1];
+      const float f = factor[s];
+      if (f != 0.f) o += f * part_o[(at0 + (size_t)s * LA_ROWS) * rank + d];
     }
-    bf16* orow = out + ((size_t)(start + flat / nh) * nh + flat % nh) * rank;
-    for (int d = threadIdx.x; d < rank; d += blockDim.x) {
-      float o = 0.f;
-      for (int s = 0; s < n_splits; ++s) {
-        const size_t at = at0 + (size_t)s * LA_ROWS;
-        const float ms = part_ml[2 * at];
-        if (ms != -INFINITY) o += expf(ms - mm) * part_o[at * rank + d];
-      }
-      orow[d] = (bf16)(o / l);
-    }
+    orow[d] = (bf16)(o / l);
   }
 }
 
+// share: the four waves of a workgroup take one tile's pages in turns (few tiles: single tokens), else a tile each.
 // n_tiles: at least the number of tiles of all sequences, sum_b ceil(new tokens_b * heads / 16) (the host may not know
 // the counts: (n_tokens * heads + 15) / 16 + n_seqs bounds it).  workspace: floats for n_tiles * n_splits * 16 *
 // (rank + 2), used when n_splits > 1.
 SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                          int table_stride, const int* seq_start, const int* seq_past, int n_seqs,
                                          void* out, float* workspace, long workspace_floats, float scale, int n_tiles,
-                                         int nh, int rank, int rot, int window, int n_splits, hipStream_t stream) {
+                                         int nh, int rank, int rot, int window, int n_splits, int share,
+                                         hipStream_t stream) {
   const int R = rank + rot;
   SYN_CHECK(n_seqs > 0 && n_tiles > 0 && nh > 0, "latent_attention: empty input");
   SYN_CHECK(rank > 0 && rank % 16 == 0 && rank <= 512 && R % 16 == 0 && R <= 640,
             "latent_attention: rows of %d + %d values (multiples of 16 up to 512 and 640 together)", rank, rot);
-  SYN_CHECK(window >= 0 && n_splits >= 1, "latent_attention: window %d, %d splits", window, n_splits);
+  SYN_CHECK(window >= 0 && n_splits >= 1 && n_splits <= LA_MAX_SPLITS, "latent_attention: window %d, %d splits", window, n_splits);
   SYN_CHECK(n_splits == 1 || (workspace != nullptr && workspace_floats >= (long)n_tiles * n_splits * LA_ROWS * (rank + 2)),
             "latent_attention: a workspace of %ld floats for %d tiles in %d splits", workspace_floats, n_tiles, n_splits);
   float* part_o = workspace;
   float* part_ml = workspace ? workspace + (size_t)n_tiles * n_splits * LA_ROWS * rank : nullptr;
-  const dim3 grid((n_tiles + 3) / 4, n_splits);
+  const dim3 grid(share ? n_tiles : (n_tiles + 3) / 4, n_splits);
   const bool x32 = R % 32 == 0;
-#define SYN_LA(DT, QS, X)                                                                                             \
-  latent_attention_bf16_kernel<DT, QS, X><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,              \
+#define SYN_LA2(DT, QS, X, S)                                                                                         \
+  latent_attention_bf16_kernel<DT, QS, X, S><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,           \
       (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs, (bf16*)out, part_o, part_ml, scale,  \
       nh, rank, R, window, n_splits)
+#define SYN_LA(DT, QS, X) do { if (share) SYN_LA2(DT, QS, X, true); else SYN_LA2(DT, QS, X, false); } while (0)
   if (rank <= 128 && R <= 160) {
     if (x32) SYN_LA(8, 5, true); else SYN_LA(8, 10, false);
   } else if (rank <= 256 && R <= 320) {
@@ -252,10 +297,11 @@ SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, con
     if (x32) SYN_LA(32, 20, true); else SYN_LA(32, 40, false);
   }
 #undef SYN_LA
+#undef SYN_LA2
   SYN_LAUNCH_CHECK("latent_attention");
   if (n_splits > 1) {
-    latent_attention_merge_kernel<<<(n_tiles + 3) / 4 * 4, 256, 0, stream>>>(part_o, part_ml, seq_start, n_seqs,
-                                                                             (bf16*)out, nh, rank, n_splits);
+    latent_attention_merge_kernel<<<dim3((n_tiles + 3) / 4 * 4, LA_ROWS), 256, 0, stream>>>(part_o, part_ml, seq_start, n_seqs,
+                                                                                            (bf16*)out, nh, rank, n_splits);
     SYN_LAUNCH_CHECK("latent_attention_merge");
   }
   return 0;

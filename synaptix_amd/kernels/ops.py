@@ -1102,7 +1102,7 @@ def _grouped(name, a, lda, a_group, w, w_group, ldw, out, ldo, o_group, M, N, K,
     _call(load_library("core"), "syn_grouped_product", _ptr(a), L(lda), L(a_group), _ptr(w), L(w_group), L(ldw), _ptr(out),
           L(ldo), L(o_group), _is_f32(a), _is_f32(out), _ptr(seg), _ptr(a_rows), _ptr(o_rows), _ptr(row_weight), _ptr(gate),
           L(gate_ld), L(gate_group), int(gate_col), int(act), int(M), int(N), int(K), int(groups), int(rows_bound),
-          int(bool(force_simt)), _stream())
+          int(force_simt), _stream())
 
 
 def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force_simt=False):
@@ -1131,13 +1131,12 @@ def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force
 ROUTE_MAX_EXPERTS, ROUTE_MAX_TOP = 1024, 64
 
 
-def route_topk(x, w, bias, ids, weights):
-    """Router of a mixture of experts: z = x . w^T + bias in 32-bit; ids [N, top] int32 the experts with the largest
-    logits (largest first, the lower index of equal ones), weights [N, top] float the softmax over those logits."""
-    _need(x, "route_topk.x", (_BF16, _F32), (None, None))
-    N, H = x.shape
-    _need(w, "route_topk.w", x.dtype, (None, H))
-    E = w.shape[0]
+def route_topk(logits, bias, ids, weights):
+    """The choice of a mixture's router: logits [N, E] float (the 32-bit sums of the router's product) + bias [E];
+    ids [N, top] int32 the experts with the largest logits (largest first, the lower index of equal ones), weights
+    [N, top] float the softmax over those logits alone."""
+    _need(logits, "route_topk.logits", _F32, (None, None))
+    N, E = logits.shape
     if bias is not None:
         _need(bias, "route_topk.bias", _F32, (E,))
     _need(ids, "route_topk.ids", _I32, (N, None))
@@ -1145,8 +1144,7 @@ def route_topk(x, w, bias, ids, weights):
     _need(weights, "route_topk.weights", _F32, (N, top))
     if not (0 < top <= min(E, ROUTE_MAX_TOP)) or E > ROUTE_MAX_EXPERTS:
         raise KernelError(f"route_topk: the {top} largest of {E} experts (at most {ROUTE_MAX_TOP} of {ROUTE_MAX_EXPERTS})")
-    _call(load_library("core"), "syn_route_topk", _ptr(x), _ptr(w), _is_f32(x), _ptr(bias), _ptr(ids), _ptr(weights), N, H,
-          E, top, _stream())
+    _call(load_library("core"), "syn_route_topk", _ptr(logits), _ptr(bias), _ptr(ids), _ptr(weights), N, E, top, _stream())
 
 
 def route_sort(ids, weights, n_experts):
@@ -1188,13 +1186,30 @@ def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False,
 
 # ----------------------------------------------------------------------------- latent attention: intake
 
+def latent_v_pages_to_kernel_order(v):
+    """Value pages [..., rank, 64] of latent attention from plain rows into the order of the bf16 kernel's fragments
+    (csrc/latent_attention.hip, la_v_offset); for tests and tools, on any device."""
+    rank = v.shape[-2]
+    if rank % 16 or v.shape[-1] != PAGE_TOKENS:
+        raise KernelError(f"latent_v_pages_to_kernel_order: pages of {rank} x {v.shape[-1]}")
+    d = torch.arange(rank, device=v.device)[:, None]
+    slot = torch.arange(PAGE_TOKENS, device=v.device)[None, :]
+    half, s = slot >> 5, slot & 31
+    e = (s & 3) + 4 * (s >> 4)
+    offset = (((((d >> 4) * 2 + half) * 64 + ((s & 15) >> 2) * 16 + (d & 15)) << 3) + e).reshape(-1)
+    out = torch.empty_like(v).reshape(*v.shape[:-2], rank * PAGE_TOKENS)
+    out[..., offset] = v.reshape(*v.shape[:-2], rank * PAGE_TOKENS)
+    return out.reshape(v.shape)
+
+
 def latent_intake(proj, gain, eps, cos, sin, q_nope, q_full, k_pages, v_pages, page_table, tok_seq, tok_pos,
-                  n_heads, dim, rot_dim, rank, max_position, write_kv=True):
+                  n_heads, dim, rot_dim, rank, max_position, write_kv=True, v_fragments=False):
     """From the fused projection proj [N, >= heads * (dim + rot_dim) + rank + rot_dim] float: q_nope [N, heads * dim];
     the rotated query parts into q_full [N, heads * (rank + rot_dim)] behind each head's first `rank` places; the
     token's cache row [RMSNorm(latent) * gain | rotated key part] into k_pages [pages, 1, 64, rank + rot_dim] and the
     normed latent as its value into v_pages [pages, 1, rank, 64].  cos, sin [capacity, pairs]: pairs (2i, 2i + 1) of
-    the rotated parts are turned, what lies behind 2 * pairs passes."""
+    the rotated parts are turned, what lies behind 2 * pairs passes.  v_fragments: the value pages are kept in the order
+    of the bf16 attention kernel's fragments (what latent_attention reads when it runs in tiles)."""
     _need(proj, "latent_intake.proj", _F32, (None, None))
     N, width = proj.shape
     R = rank + rot_dim
@@ -1218,7 +1233,7 @@ def latent_intake(proj, gain, eps, cos, sin, q_nope, q_full, k_pages, v_pages, p
     _call(load_library("core"), "syn_latent_intake", _ptr(proj), width, _ptr(gain), _is_f32(gain), ctypes.c_float(eps),
           _ptr(cos), _ptr(sin), n_pairs, capacity, int(max_position), _ptr(q_nope), _ptr(q_full), _ptr(k_pages),
           _ptr(v_pages), _is_f32(q_nope), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), N, n_heads,
-          dim, rot_dim, rank, int(bool(write_kv)), _stream())
+          dim, rot_dim, rank, int(bool(write_kv)), int(bool(v_fragments)), _stream())
 
 
 # ----------------------------------------------------------------------------- latent attention
@@ -1240,15 +1255,19 @@ def latent_attention_takes(rank, rot_dim, dtype=_F32) -> bool:
 
 
 def _latent_tiles(n_tokens, n_heads, n_seqs, max_pages):
-    """(a bound on the tiles of 16 (token, head) rows, the splits of a tile's pages): many tiles run whole, few are cut
-    until some 2,048 waves have work."""
+    """(a bound on the tiles of 16 (token, head) rows, the splits of a tile's pages, whether a workgroup's waves share a
+    tile): many tiles run whole, a wave each."""
     tiles = (n_tokens * n_heads + 15) // 16 + n_seqs
-    return tiles, max(1, min(int(max_pages), 2048 // tiles))
+    if tiles >= 256:
+        return tiles, 1, False
+    # few tiles: the four waves of a workgroup share a tile's pages, and the pages are cut further until some 1,024
+    # workgroups have work
+    return tiles, max(1, min((int(max_pages) + 3) // 4, 1024 // tiles, 1024)), True
 
 
 def latent_attention_workspace(n_tokens, n_heads, n_seqs, rank, max_pages) -> int:
     """Floats of workspace that latent_attention needs for a step of these sizes (0: none)."""
-    tiles, splits = _latent_tiles(n_tokens, n_heads, n_seqs, max_pages)
+    tiles, splits, _ = _latent_tiles(n_tokens, n_heads, n_seqs, max_pages)
     return tiles * splits * 16 * (rank + 2) if splits > 1 else 0
 
 
@@ -1260,7 +1279,9 @@ def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out
     k_j[:rank] over the keys at or before the query's position (window > 0: the last `window` of them).  Scores,
     weights and sums are 32-bit.  seqs = (seq_start [B + 1], seq_past [B]): the step's sequences, whose new tokens lie
     one after another at positions seq_past[b] ..; with them bf16 runs in tiles on the matrix cores where the sizes
-    allow (latent_attention_tiled), with `workspace` floats (latent_attention_workspace) for tiles cut into splits."""
+    allow (latent_attention_tiled), with `workspace` floats (latent_attention_workspace) for tiles cut into splits; the
+    value pages are then in the order of that kernel's fragments (latent_intake(v_fragments=True),
+    latent_v_pages_to_kernel_order)."""
     R = rank + rot_dim
     if q_full.dtype == _BF16 and seqs is not None and latent_attention_tiled(rank, rot_dim) and not force_simt:
         seq_start, seq_past = seqs
@@ -1275,7 +1296,7 @@ def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out
         if page_table.shape[0] < B:
             raise KernelError(f"latent_attention: page table has {page_table.shape[0]} rows for {B} sequences")
         _need(out, "latent_attention.out", _BF16, (N, n_heads * rank))
-        tiles, splits = _latent_tiles(N, n_heads, B, page_table.shape[1])
+        tiles, splits, share = _latent_tiles(N, n_heads, B, page_table.shape[1])
         floats = 0
         if splits > 1:
             need = tiles * splits * 16 * (rank + 2)
@@ -1287,6 +1308,6 @@ def latent_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out
                 raise KernelError(f"latent_attention: a workspace of {floats} floats, {need} needed")
         _call(load_library("core"), "syn_latent_attention_bf16", _ptr(q_full), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
               page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, _ptr(out), _ptr(workspace if splits > 1 else None),
-              ctypes.c_long(floats), ctypes.c_float(scale), tiles, n_heads, rank, rot_dim, int(window or 0), splits, _stream())
+              ctypes.c_long(floats), ctypes.c_float(scale), tiles, n_heads, rank, rot_dim, int(window or 0), splits, int(share), _stream())
         return
     window_attention(q_full, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, 1, R, rank, window=window)

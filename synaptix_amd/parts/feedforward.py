@@ -75,7 +75,8 @@ class GatedMlp(FeedForward):
 class RoutedExperts(FeedForward):
     """A mixture of small ungated experts: each token goes through the `top` experts whose router logits are largest,
 
-        z = W_router h + b (32-bit);   chosen: the `top` largest z;   weights: softmax over the chosen logits only
+        z = W_router h + b (32-bit sums of the framework's own product);   chosen: the `top` largest z;
+        weights: softmax over the chosen logits only
         y = sum_chosen weight_e * W_down[e] act(W_up[e] h)
 
     The tokens are sorted by expert on the device (no count comes back to the host), and each expert's rows meet its
@@ -111,7 +112,7 @@ class RoutedExperts(FeedForward):
         p, (up, down, router, bias) = self.prefix, self.names
         self.w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
         self.w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
-        self.w_router = get(p + router)
+        self.w_router = Matrix(get(p + router))
         self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
 
     def check(self, dtype):
@@ -124,7 +125,7 @@ class RoutedExperts(FeedForward):
         N, dev = h.shape[0], h.device
         ids = torch.empty((N, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((N, self.top), dtype=torch.float32, device=dev)
-        ops.route_topk(h, self.w_router, self.b_router, ids, weights)
+        ops.route_topk(linear(h, self.w_router, torch.float32), self.b_router, ids, weights)
         seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, self.n_experts)
         mid = torch.empty((N * self.top, self.ff), dtype=h.dtype, device=dev)
         ops.experts_product(h, self.w_up, mid, seg, tok_of, pair_of, gelu=True)

@@ -103,14 +103,16 @@ class LatentAttention(Mixer):
         q_full = torch.empty((N, nh * R), dtype=act, device=dev)
         cos, sin = self.position.tables(dev)
         table = ctx.page_table(cache.group)
+        # (bf16 whose sizes the tiles on the matrix cores take: the value pages lie in that kernel's order)
+        tiled = act == torch.bfloat16 and ops.latent_attention_tiled(rank, rot)
         ops.latent_intake(proj, self.gain, self.norm_eps, cos, sin, q_nope, q_full, cache.k_pages, cache.v_pages, table,
-                          ctx.tok_seq, ctx.tok_pos, nh, dim, rot, rank, ctx.max_position, write_kv=owner)
+                          ctx.tok_seq, ctx.tok_pos, nh, dim, rot, rank, ctx.max_position, write_kv=owner, v_fragments=tiled)
         # the query in the latent's space, into the first `rank` places of each head's row
         ops.heads_product(q_nope.view(N, nh, dim), self.w_uk_t, q_full.view(N, nh, R))
         o_lat = torch.empty((N, nh * rank), dtype=act, device=dev)
-        floats = ops.latent_attention_workspace(N, nh, ctx.n_seqs, rank, table.shape[1]) if act == torch.bfloat16 else 0
+        floats = ops.latent_attention_workspace(N, nh, ctx.n_seqs, rank, table.shape[1]) if tiled else 0
         ops.latent_attention(q_full, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o_lat, self.scale, nh,
-                             rank, rot, window=self.window or 0, seqs=(ctx.seq_start, ctx.seq_past),
+                             rank, rot, window=self.window or 0, seqs=(ctx.seq_start, ctx.seq_past) if tiled else None,
                              workspace=ctx.scratch("latent_attention", floats) if floats else None)
         o = torch.empty((N, nh * vdim), dtype=act, device=dev)
         gate = proj[:, nh * (dim + rot) + R:] if self.gate else None

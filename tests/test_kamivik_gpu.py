@@ -64,10 +64,12 @@ def test_scaled_terms_into_the_residual_and_the_norm(W):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("N,H,K,J", [(70, 3, 32, 40), (5, 2, 64, 16), (33, 4, 20, 7), (1, 1, 96, 130), (130, 2, 128, 64)])
+@pytest.mark.parametrize("N,H,K,J", [(70, 3, 32, 40), (5, 2, 64, 16), (33, 4, 20, 7), (1, 1, 96, 130), (130, 2, 128, 64),
+                                     (100, 2, 40, 24), (300, 1, 72, 200)])
 def test_a_linear_map_for_each_head(N, H, K, J, dtype):
-    """On the matrix cores where K is a multiple of 32 (bf16), in plain FMA otherwise; into a piece of longer rows;
-    with one gate a head and with one gate a value."""
+    """In bf16 on the matrix cores: tiles through LDS from 48 rows on (any K that is a multiple of 8, a last k-tile
+    that is partly empty), operands straight from memory for fewer rows (K a multiple of 32); plain FMA otherwise;
+    into a piece of longer rows; with one gate a head and with one gate a value."""
     from synaptix_amd.kernels import ops
     g = torch.Generator().manual_seed(N + K)
     x, w = rounded(dtype, torch.randn(N, H, K, generator=g), torch.randn(H, J, K, generator=g) / math.sqrt(K))
@@ -84,15 +86,16 @@ def test_a_linear_map_for_each_head(N, H, K, J, dtype):
     assert float((out.cpu().double() - plain * torch.sigmoid(gate[:, 3:]).view(N, H, J)).abs().max()) < tol
     ops.heads_product(dev(x, dtype), dev(w, dtype), out, gate=G[:, 1:1 + H], gate_per_value=False)
     assert float((out.cpu().double() - plain * torch.sigmoid(gate[:, 1:1 + H])[:, :, None]).abs().max()) < tol
-    if dtype == torch.bfloat16:           # both kernels give the sums of the same products
-        other = torch.empty_like(out)
-        ops.heads_product(dev(x, dtype), dev(w, dtype), other, gate=G[:, 1:1 + H], gate_per_value=False, force_simt=True)
-        assert float((other.float() - out.float()).abs().max()) < tol
+    if dtype == torch.bfloat16:           # all kernels give the sums of the same products
+        for force in (1, 2):              # plain FMA; the matrix cores without LDS (where K allows, else FMA again)
+            other = torch.empty_like(out)
+            ops.heads_product(dev(x, dtype), dev(w, dtype), other, gate=G[:, 1:1 + H], gate_per_value=False, force_simt=force)
+            assert float((other.float() - out.float()).abs().max()) < tol
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("N,W,F,E,top", [(50, 64, 32, 6, 2), (3, 40, 24, 5, 5), (1, 32, 96, 4, 1), (200, 96, 64, 16, 3),
-                                         (9, 72, 20, 1, 1)])
+                                         (9, 72, 20, 1, 1), (300, 64, 40, 4, 2)])
 def test_router_and_experts(N, W, F, E, top, dtype):
     """The router's logits are spread so that no choice is close; an expert that nobody chose has an empty segment."""
     from synaptix_amd.kernels import ops
@@ -105,7 +108,8 @@ def test_router_and_experts(N, W, F, E, top, dtype):
     want_ids, want_w = P.route(h, wr, bias, top)
     ids = torch.empty((N, top), dtype=torch.int32, device=DEV)
     weights = torch.empty((N, top), dtype=torch.float32, device=DEV)
-    ops.route_topk(dev(h, dtype), dev(wr, dtype), dev(bias), ids, weights)
+    from synaptix_amd.parts import linear, Matrix
+    ops.route_topk(linear(dev(h, dtype), Matrix(dev(wr, dtype)), torch.float32), dev(bias), ids, weights)
     assert torch.equal(ids.cpu().long(), want_ids)
     assert float((weights.cpu().double() - want_w).abs().max()) < 1e-4
     seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, E)
@@ -120,7 +124,7 @@ def test_router_and_experts(N, W, F, E, top, dtype):
     for t in range(N):
         for e, a in zip(want_ids[t].tolist(), want_w[t]):
             want[t] += a * (downs[e] @ P.gelu(ups[e] @ h[t]))
-    for force in (False, True):
+    for force in (0, 1, 2):
         mid = torch.empty((N * top, F), dtype=dtype, device=DEV)
         ops.experts_product(dev(h, dtype), dev(ups, dtype), mid, seg, tok_of, pair_of, gelu=True, force_simt=force)
         y = torch.empty((top, N, W), dtype=torch.float32, device=DEV)
@@ -188,12 +192,12 @@ def test_latent_attention_sees_exactly_its_keys(window, dtype):
 @pytest.mark.parametrize("window", [0, 1, 64, 65, 130])
 def test_latent_attention_in_tiles_on_the_matrix_cores(window, H, C, B):
     """The bf16 kernel whose tiles are 16 (token, head) rows of one sequence, for every size of its register tiles, with
-    k-steps of 16 and of 32: two sequences in one step, the second continuing from 70 cached rows (a portion that
+    k-steps of 16 and of 32: two sequences in one step, the second (470 rows) continuing from 70 cached rows (a portion that
     starts inside a page); then single tokens of both sequences together, whose pages are cut into splits and merged.
     Rows and queries as in the test above (a wrong or lost key shows); slots behind a sequence's end hold NaN."""
     from synaptix_amd.kernels import ops
     R, dt = C + B, torch.bfloat16
-    lens, past = [150, 210], [0, 70]
+    lens, past = [150, 470], [0, 70]
     g = torch.Generator().manual_seed(window + H)
     qs, rowss, wants = [], [], []
     for T in lens:
@@ -221,7 +225,7 @@ def test_latent_attention_in_tiles_on_the_matrix_cores(window, H, C, B):
         last, used = int(table[j, (lens[j] - 1) // 64]), (lens[j] - 1) % 64 + 1
         kp[last, 0, used:] = float("nan")
         vp[last, 0, :, used:] = float("nan")
-    kp, vp = kp.to(dt), vp.to(dt)
+    kp, vp = kp.to(dt), ops.latent_v_pages_to_kernel_order(vp.to(dt))
     new = [lens[0] - past[0], lens[1] - past[1]]
     q_step = torch.cat([qs[0][past[0]:], qs[1][past[1]:]]).reshape(-1, H * R)
     want = torch.cat([wants[0][past[0]:], wants[1][past[1]:]])
@@ -277,6 +281,12 @@ def test_latent_intake_norms_turns_and_writes_the_pages(H, D, B, C, pairs, dtype
         assert float((kp[page, 0, slot].cpu().double() - want_row[n]).abs().max()) < tol
         assert float((vp[page, 0, :, slot].cpu().double() - want_row[n, :C]).abs().max()) < tol
     assert int((kp.float().abs().sum(-1) > 0).sum()) == N                # nothing else was written
+    if C % 16 == 0:           # the value pages in the order of the bf16 attention kernel's fragments
+        vf = torch.zeros_like(vp)
+        ops.latent_intake(dev(proj), dev(gain), 1e-5, cos, sin, qn, qf, kp, vf, table,
+                          torch.tensor(seqs, dtype=torch.int32, device=DEV), torch.tensor(pos, dtype=torch.int32, device=DEV),
+                          H, D, B, C, max(pos), v_fragments=True)
+        assert torch.equal(vf, ops.latent_v_pages_to_kernel_order(vp))
 
 
 # ----------------------------------------------------------------------------- whole models
