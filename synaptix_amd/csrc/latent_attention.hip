@@ -57,8 +57,26 @@ __host__ __device__ __forceinline__ int la_v_offset(int d, int slot) {
   return ((((d >> 4) * 2 + half) * 64 + g * 16 + (d & 15)) << 3) + e;
 }
 
+// the sequence and the unit inside it of global unit t, a unit being `unit_rows` consecutive (token, head) rows
+__device__ __forceinline__ bool la_find_unit(int t, int unit_rows, const int* seq_start, int n_seqs, int nh, int& seq,
+                                             int& unit, int& start, int& rows) {
+  for (int b = 0; b < n_seqs; ++b) {
+    const int s0 = seq_start[b], n = (seq_start[b + 1] - s0) * nh, units = (n + unit_rows - 1) / unit_rows;
+    if (t < units) {
+      seq = b, unit = t, start = s0, rows = n;
+      return true;
+    }
+    t -= units;
+  }
+  return false;
+}
+
 // DT: tiles of 16 values that the accumulators hold (rank <= 16 DT); QS: k-steps that the query's registers hold
 // (R <= QS * (X32 ? 32 : 16)); X32: k-steps of 32 (R a multiple of 32) or of 16.
+// SHARE false (prompts): a workgroup takes four consecutive tiles of one sequence, a wave each, and walks the pages
+// that any of them sees: a page's keys and values go through LDS once for the four (rows of keys padded by 16 bytes
+// against bank conflicts; dynamic LDS: 64 (R + 8) + 64 rank bf16 values).  SHARE true (single tokens): a workgroup
+// takes one tile, its waves the tile's pages in turns, operands straight from memory, merged through LDS at the end.
 template <int DT, int QS, bool X32, bool SHARE>
 __global__ void __launch_bounds__(256)
 latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
@@ -68,23 +86,22 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
                              int window, int n_splits) {
   typedef typename LaFrag<X32>::type frag;
   constexpr int KS = X32 ? 32 : 16, PIECE = KS / 4;
+  extern __shared__ __attribute__((aligned(16))) bf16 la_stage[];      // (SHARE false) a page's keys, then its values
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, g = lane / 16;
-  // SHARE: the workgroup's waves take one tile's pages in turns; else a tile a wave
-  const int gt = SHARE ? blockIdx.x : blockIdx.x * 4 + wave, split = blockIdx.y;
-  int seq, tile, start, rows;
-  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;      // (SHARE: the whole workgroup)
+  const int split = blockIdx.y;
+  int seq, unit, start, rows;
+  if (!la_find_unit(blockIdx.x, SHARE ? LA_ROWS : 4 * LA_ROWS, seq_start, n_seqs, nh, seq, unit, start, rows)) return;
+  const int tile = SHARE ? unit : unit * 4 + wave;
+  const bool tile_ok = tile * LA_ROWS < rows;                            // (SHARE: always)
   const int past = seq_past[seq];
-  const int flat0 = tile * LA_ROWS, flat_last = min(flat0 + LA_ROWS, rows) - 1;
-  const bool row_ok = flat0 + i < rows;
+  const int flat0 = tile_ok ? tile * LA_ROWS : rows - 1, flat_last = min(flat0 + LA_ROWS, rows) - 1;
+  const bool row_ok = tile_ok && flat0 + i < rows;
   const int flat = row_ok ? flat0 + i : flat_last;       // a row beyond the tile's end repeats the last one, unstored
   const int tok = flat / nh, head = flat % nh, pos = past + tok;
   const int kv_len = past + rows / nh;
-  // the pages that some row of the tile sees, and this split's share of them
+  // the pages that some row of the tile sees
   const int pos_lo = past + flat0 / nh, pos_hi = past + flat_last / nh;
-  const int key_lo = window > 0 ? max(0, pos_lo - window + 1) : 0;
-  const int page_lo = key_lo / SYN_PAGE, page_hi = pos_hi / SYN_PAGE;
-  const int chunk = (page_hi - page_lo + n_splits) / n_splits;
-  const int p0 = page_lo + split * chunk, p1 = min(p0 + chunk, page_hi + 1);
+  const int my_lo = (window > 0 ? max(0, pos_lo - window + 1) : 0) / SYN_PAGE, my_hi = pos_hi / SYN_PAGE;
   const int n_qs = R / KS, n_dt = rank / 16;
 
   frag qf[QS];
@@ -98,9 +115,10 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int* pages = page_table + (size_t)seq * table_stride;
-  for (int p = SHARE ? p0 + wave : p0; p < p1; p += SHARE ? 4 : 1) {
-    const int page = pages[p];
-    const bf16* kb = k_pages + (size_t)page * SYN_PAGE * R + (size_t)i * R + g * PIECE;
+
+  // one page of 64 keys against the tile: kb = the lane's place in the page's first key row (rows of k_ld values),
+  // vb = the lane's place in the page's first value fragment
+  auto one_page = [&](const bf16* kb, int k_ld, const bf16* vb, int p) {
     f32x4 s[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -109,7 +127,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
       if (ks < n_qs) {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-          const frag a = *(const frag*)(kb + (size_t)kt * 16 * R + ks * KS);
+          const frag a = *(const frag*)(kb + kt * 16 * k_ld + ks * KS);
           s[kt] = la_mfma(a, qf[ks], s[kt]);
         }
       }
@@ -150,7 +168,6 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
       if (dt < n_dt) acc[dt] *= alpha;
     // slots behind the sequence's end may hold anything: their weights are 0, their values are made 0 as well
     const int left = kv_len - p * SYN_PAGE;
-    const bf16* vb = v_pages + (size_t)page * rank * SYN_PAGE + lane * 8;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       bf16x8 ph, pl;
@@ -174,6 +191,43 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
           acc[dt] = la_mfma(a, pl, acc[dt]);
         }
     }
+  };
+
+  if constexpr (SHARE) {
+    // this split's share of the tile's pages, a page a wave in turns, operands straight from memory
+    const int chunk = (my_hi - my_lo + n_splits) / n_splits;
+    const int p0 = my_lo + split * chunk, p1 = min(p0 + chunk, my_hi + 1);
+    for (int p = p0 + wave; p < p1; p += 4) {
+      const int page = pages[p];
+      one_page(k_pages + (size_t)page * SYN_PAGE * R + (size_t)i * R + g * PIECE, R,
+               v_pages + (size_t)page * rank * SYN_PAGE + lane * 8, p);
+    }
+  } else {
+    // the pages that any of the workgroup's four tiles sees, each through LDS once
+    const int k_ld = R + 8;
+    bf16* ks_ = la_stage;
+    bf16* vs_ = la_stage + SYN_PAGE * k_ld;
+    const int g_first = unit * 4 * LA_ROWS, g_last = min(g_first + 4 * LA_ROWS, rows) - 1;
+    const int g_lo = (window > 0 ? max(0, past + g_first / nh - window + 1) : 0) / SYN_PAGE;
+    const int g_hi = (past + g_last / nh) / SYN_PAGE;
+    const int cpr = R / 8;                                   // 16-byte chunks of a key row
+    const int row_step = 256 / cpr, col_step = 256 % cpr;
+    for (int p = g_lo; p <= g_hi; ++p) {
+      const int page = pages[p];
+      const bf16* ksrc = k_pages + (size_t)page * SYN_PAGE * R;
+      const bf16* vsrc = v_pages + (size_t)page * rank * SYN_PAGE;
+      __syncthreads();                                       // everybody has done with the page before
+      int row = threadIdx.x / cpr, col = threadIdx.x % cpr;
+      for (int c = threadIdx.x; c < SYN_PAGE * cpr; c += 256) {
+        *(bf16x8*)(ks_ + row * k_ld + col * 8) = *(const bf16x8*)(ksrc + (size_t)c * 8);
+        row += row_step, col += col_step;
+        if (col >= cpr) col -= cpr, ++row;
+      }
+      for (int c = threadIdx.x; c < rank * 8; c += 256) *(bf16x8*)(vs_ + c * 8) = *(const bf16x8*)(vsrc + (size_t)c * 8);
+      __syncthreads();
+      if (tile_ok && p >= my_lo && p <= my_hi) one_page(ks_ + i * k_ld + g * PIECE, k_ld, vs_ + lane * 8, p);
+    }
+    if (!tile_ok) return;
   }
   // acc[dt][e]: value dt * 16 + 4 g + e of this lane's row
   if constexpr (SHARE) {
@@ -218,7 +272,8 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         *(bf16x4*)(orow + dt * 16) = r;
       }
   } else {
-    const size_t at = ((size_t)gt * n_splits + split) * LA_ROWS + i;
+    // (SHARE only: blockIdx.x is the tile's number among all tiles)
+    const size_t at = ((size_t)blockIdx.x * n_splits + split) * LA_ROWS + i;
     if (g == 0) part_ml[2 * at] = m, part_ml[2 * at + 1] = l;
     float* prow = part_o + at * rank + 4 * g;
 #pragma unroll
@@ -264,8 +319,30 @@ latent_attention_merge_kernel(const float* __restrict__ part_o, const float* __r
   }
 }
 
-// share: the four waves of a workgroup take one tile's pages in turns (few tiles: single tokens), else a tile each.
-// n_tiles: at least the number of tiles of all sequences, sum_b ceil(new tokens_b * heads / 16) (the host may not know
+template <int DT, int QS, bool X32, bool SHARE>
+static int la_launch(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int table_stride,
+                     const int* seq_start, const int* seq_past, int n_seqs, void* out, float* part_o, float* part_ml,
+                     float scale, int n_tiles, int nh, int rank, int R, int window, int n_splits, hipStream_t stream) {
+  // SHARE: a workgroup a tile; else a workgroup for every four tiles of a sequence (n_tiles bounds both counts)
+  const dim3 grid(n_tiles, n_splits);
+  const size_t lds = SHARE ? 0 : ((size_t)SYN_PAGE * (R + 8) + (size_t)SYN_PAGE * rank) * sizeof(bf16);
+  static OncePerDevice raised;
+  if (lds > 49152) {
+    const hipError_t e = once_per_device(raised, [&] {
+      return hipFuncSetAttribute((const void*)latent_attention_bf16_kernel<DT, QS, X32, SHARE>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+    });
+    SYN_CHECK(e == hipSuccess, "latent_attention: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+  }
+  latent_attention_bf16_kernel<DT, QS, X32, SHARE><<<grid, 256, lds, stream>>>(
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
+      (bf16*)out, part_o, part_ml, scale, nh, rank, R, window, n_splits);
+  return 0;
+}
+
+// share: the four waves of a workgroup take one tile's pages in turns (few tiles: single tokens), else a tile each
+// and no splits.  n_tiles: the workgroups, at least the number of all sequences' tiles (share) or groups of four tiles;
+// with share at least the number of tiles of all sequences, sum_b ceil(new tokens_b * heads / 16) (the host may not know
 // the counts: (n_tokens * heads + 15) / 16 + n_seqs bounds it).  workspace: floats for n_tiles * n_splits * 16 *
 // (rank + 2), used when n_splits > 1.
 SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
@@ -280,15 +357,16 @@ SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, con
   SYN_CHECK(window >= 0 && n_splits >= 1 && n_splits <= LA_MAX_SPLITS, "latent_attention: window %d, %d splits", window, n_splits);
   SYN_CHECK(n_splits == 1 || (workspace != nullptr && workspace_floats >= (long)n_tiles * n_splits * LA_ROWS * (rank + 2)),
             "latent_attention: a workspace of %ld floats for %d tiles in %d splits", workspace_floats, n_tiles, n_splits);
+  SYN_CHECK(share || n_splits == 1, "latent_attention: pages are cut into splits only where a workgroup shares a tile");
   float* part_o = workspace;
   float* part_ml = workspace ? workspace + (size_t)n_tiles * n_splits * LA_ROWS * rank : nullptr;
-  const dim3 grid(share ? n_tiles : (n_tiles + 3) / 4, n_splits);
   const bool x32 = R % 32 == 0;
-#define SYN_LA2(DT, QS, X, S)                                                                                         \
-  latent_attention_bf16_kernel<DT, QS, X, S><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,           \
-      (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs, (bf16*)out, part_o, part_ml, scale,  \
-      nh, rank, R, window, n_splits)
-#define SYN_LA(DT, QS, X) do { if (share) SYN_LA2(DT, QS, X, true); else SYN_LA2(DT, QS, X, false); } while (0)
+  int rc = 0;
+#define SYN_LA(DT, QS, X)                                                                                          \
+  rc = share ? la_launch<DT, QS, X, true>(q, k_pages, v_pages, page_table, table_stride, seq_start, seq_past, n_seqs, \
+                                          out, part_o, part_ml, scale, n_tiles, nh, rank, R, window, n_splits, stream) \
+             : la_launch<DT, QS, X, false>(q, k_pages, v_pages, page_table, table_stride, seq_start, seq_past, n_seqs, \
+                                           out, part_o, part_ml, scale, n_tiles, nh, rank, R, window, n_splits, stream)
   if (rank <= 128 && R <= 160) {
     if (x32) SYN_LA(8, 5, true); else SYN_LA(8, 10, false);
   } else if (rank <= 256 && R <= 320) {
@@ -297,7 +375,7 @@ SYN_EXPORT int syn_latent_attention_bf16(const void* q, const void* k_pages, con
     if (x32) SYN_LA(32, 20, true); else SYN_LA(32, 40, false);
   }
 #undef SYN_LA
-#undef SYN_LA2
+  if (rc) return rc;
   SYN_LAUNCH_CHECK("latent_attention");
   if (n_splits > 1) {
     latent_attention_merge_kernel<<<dim3((n_tiles + 3) / 4 * 4, LA_ROWS), 256, 0, stream>>>(part_o, part_ml, seq_start, n_seqs,

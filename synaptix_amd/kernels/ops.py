@@ -1255,11 +1255,12 @@ def latent_attention_takes(rank, rot_dim, dtype=_F32) -> bool:
 
 
 def _latent_tiles(n_tokens, n_heads, n_seqs, max_pages):
-    """(a bound on the tiles of 16 (token, head) rows, the splits of a tile's pages, whether a workgroup's waves share a
-    tile): many tiles run whole, a wave each."""
+    """(a bound on the workgroups, the splits of a tile's pages, whether a workgroup's waves share a tile of 16 (token,
+    head) rows): many tiles run whole, a wave each and four of a sequence a workgroup."""
     tiles = (n_tokens * n_heads + 15) // 16 + n_seqs
     if tiles >= 256:
-        return tiles, 1, False
+        # (a workgroup for every four tiles of a sequence: the bound counts those)
+        return (n_tokens * n_heads + 63) // 64 + n_seqs, 1, False
     # few tiles: the four waves of a workgroup share a tile's pages, and the pages are cut further until some 1,024
     # workgroups have work
     return tiles, max(1, min((int(max_pages) + 3) // 4, 1024 // tiles, 1024)), True
