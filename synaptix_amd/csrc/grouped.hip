@@ -94,6 +94,9 @@ __global__ void __launch_bounds__(256) grouped_product_simt_kernel(GroupedArgs g
 // Both operands are 16-byte pieces of rows (8 k-values of lane group lane / 16), so whatever order the instruction
 // gives the k-values inside a lane group, the two operands agree.
 #define GP_TM 32
+// NB: blocks of 16 outputs a wave (4: 64 outputs; 1: 16 outputs, four times the waves, where few groups have rows and
+// each group's matrix has to be streamed by more than a few waves).
+template <int NB>
 __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g) {
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, i = lane % 16, q = lane / 16;
   int b = blockIdx.z, row0, row_end;
@@ -113,43 +116,70 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
     row0 = blockIdx.x * GP_TM, row_end = g.M;
     if (row0 >= row_end) return;
   }
-  const int n0 = (blockIdx.y * 4 + wave) * 64;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * NB;
   if (n0 >= g.N) return;
   const bf16* A = (const bf16*)g.a + (size_t)b * g.a_group;
   const bf16* W = (const bf16*)g.w + (size_t)b * g.w_group;
+  // rows beyond the segment and outputs beyond N read row 0 (a valid address) and count as zeros
   const bf16* arow[2];
   bool a_ok[2];
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int r = row0 + mb * 16 + i;
     a_ok[mb] = r < row_end;
-    const int src = a_ok[mb] ? (g.a_rows ? g.a_rows[r] : r) : 0;
+    const int src = a_ok[mb] ? (g.a_rows ? g.a_rows[r] : r) : (g.a_rows ? g.a_rows[row0] : row0);
     arow[mb] = A + (size_t)src * g.lda + q * 8;
   }
-  const bf16* wrow[4];
-  bool w_ok[4];
+  const bf16* wrow[NB];
+  bool w_ok[NB];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     const int n = n0 + nb * 16 + i;
     w_ok[nb] = n < g.N;
     wrow[nb] = W + (size_t)(w_ok[nb] ? n : 0) * g.ldw + q * 8;
   }
-  f32x4 acc[2][4];
+  f32x4 acc[2][NB];
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < g.K; k0 += 32) {
-    bf16x8 xa[2], xw[4];
+  // several k-steps at a time: their loads (24) are asked for together (a group's matrix is read once, as a stream), then
+  // multiplied; the k-steps that are left over follow one by one
+  constexpr int AHEAD = NB == 1 ? 8 : 4;
+  int k0 = 0;
+  for (; k0 + 32 * AHEAD <= g.K; k0 += 32 * AHEAD) {
+    bf16x8 xa[AHEAD][2], xw[AHEAD][NB];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) xa[u][mb] = *(const bf16x8*)(arow[mb] + k0 + 32 * u);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) xw[u][nb] = __builtin_nontemporal_load((const bf16x8*)(wrow[nb] + k0 + 32 * u));
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) xa[u][mb] = a_ok[mb] ? xa[u][mb] : zero;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) xw[u][nb] = w_ok[nb] ? xw[u][nb] : zero;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xw[u][nb], xa[u][mb], acc[mb][nb], 0, 0, 0);
+    }
+  }
+  for (; k0 < g.K; k0 += 32) {
+    bf16x8 xa[2], xw[NB];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) xa[mb] = a_ok[mb] ? *(const bf16x8*)(arow[mb] + k0) : zero;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) xw[nb] = w_ok[nb] ? *(const bf16x8*)(wrow[nb] + k0) : zero;
+    for (int nb = 0; nb < NB; ++nb) xw[nb] = w_ok[nb] ? *(const bf16x8*)(wrow[nb] + k0) : zero;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
+      for (int nb = 0; nb < NB; ++nb)
         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xw[nb], xa[mb], acc[mb][nb], 0, 0, 0);
   }
 #pragma unroll
@@ -157,7 +187,7 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
     const int r = row0 + mb * 16 + i;
     if (r >= row_end) continue;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int n = n0 + nb * 16 + q * 4 + e;
@@ -167,20 +197,26 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
 }
 
 // ---------------------------------------------------------------- bf16 on the matrix cores, many rows a group
-// Tiles of 128 rows x 128 outputs x 32 k through LDS (double-buffered: while one k-tile is multiplied the next is on
+// Tiles of 128 rows x 128 outputs x 64 k through LDS (double-buffered: while one k-tile is multiplied the next is on
 // its way from memory into registers), four waves of 64 x 64 each, MFMA 32x32x16: A = rows of x, B = rows of W,
 // D[m = 8 (e / 4) + 4 (lane / 32) + e % 4][n = lane % 32].  Rows of x are gathered through a_rows on their way into
 // LDS.  K is a multiple of 8 (a 16-byte chunk lies inside or outside as a whole).
 #define GT_BM 128
 #define GT_BN 128
-#define GT_BK 32
+#define GT_BK 64
 #define GT_LD (GT_BK + 8)
 __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs g) {
-  __shared__ __attribute__((aligned(16))) bf16 smem[2 * (GT_BM + GT_BN) * GT_LD];
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];      // [2][(GT_BM + GT_BN) * GT_LD]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  // Workgroups go to the eight XCDs in turns, each with an L2 of its own: workgroup w takes place
+  // (w % 8) * (places / 8) + w / 8 of the order (row tile, column tile), so that one XCD walks the column tiles of a
+  // few row tiles: it reads those rows of x once, and a group's matrix for the group's few row tiles in a row.
+  const int col_tiles = (g.N + GT_BN - 1) / GT_BN;
+  const int places = gridDim.x;                       // a multiple of 8
+  const int place = (blockIdx.x % 8) * (places / 8) + blockIdx.x / 8;
   int b = blockIdx.z, row0, row_end;
   if (g.seg_start) {
-    int t = blockIdx.x;
+    int t = place / col_tiles;
     b = -1;
     for (int e = 0; e < g.groups; ++e) {
       const int s0 = g.seg_start[e], n = g.seg_start[e + 1] - s0, tiles = (n + GT_BM - 1) / GT_BM;
@@ -192,10 +228,10 @@ __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs 
     }
     if (b < 0) return;                      // (the whole workgroup, before any barrier)
   } else {
-    row0 = blockIdx.x * GT_BM, row_end = g.M;
+    row0 = (place / col_tiles) * GT_BM, row_end = g.M;
     if (row0 >= row_end) return;
   }
-  const int n0 = blockIdx.y * GT_BN;
+  const int n0 = (place % col_tiles) * GT_BN;
   const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
   constexpr int CPR = GT_BK / 8, RPP = 256 / CPR, XL = GT_BM / RPP, WL = GT_BN / RPP;
   const int lrow = tid / CPR, lchunk = (tid % CPR) * 8;
@@ -301,12 +337,25 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
                       (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
   if (!in_is_f32 && chunks && force_simt == 0 && rows_a_group >= 48) {
     const int row_tiles = seg_start ? (rows_bound + GT_BM - 1) / GT_BM + groups : (M + GT_BM - 1) / GT_BM;
-    const dim3 grid(row_tiles, (N + GT_BN - 1) / GT_BN, seg_start ? 1 : groups);
-    grouped_product_tiled_kernel<<<grid, 256, 0, stream>>>(g);
+    const int places = (row_tiles * ((N + GT_BN - 1) / GT_BN) + 7) / 8 * 8;
+    const dim3 grid(places, 1, seg_start ? 1 : groups);
+    const size_t lds = (size_t)2 * (GT_BM + GT_BN) * GT_LD * sizeof(bf16);
+    static OncePerDevice raised;
+    const hipError_t e = once_per_device(raised, [&] {
+      return hipFuncSetAttribute((const void*)grouped_product_tiled_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    SYN_CHECK(e == hipSuccess, "grouped_product: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+    grouped_product_tiled_kernel<<<grid, 256, lds, stream>>>(g);
   } else if (!in_is_f32 && aligned && force_simt != 1) {
     const int row_tiles = seg_start ? (rows_bound + GP_TM - 1) / GP_TM + groups : (M + GP_TM - 1) / GP_TM;
-    const dim3 grid(row_tiles, (N + 255) / 256, seg_start ? 1 : groups);
-    grouped_product_mfma_kernel<<<grid, 256, 0, stream>>>(g);
+    const long wide = (long)row_tiles * ((N + 255) / 256) * (seg_start ? 1 : groups);
+    if (wide >= 2L * syn_compute_units()) {
+      const dim3 grid(row_tiles, (N + 255) / 256, seg_start ? 1 : groups);
+      grouped_product_mfma_kernel<4><<<grid, 256, 0, stream>>>(g);
+    } else {
+      const dim3 grid(row_tiles, (N + 63) / 64, seg_start ? 1 : groups);
+      grouped_product_mfma_kernel<1><<<grid, 256, 0, stream>>>(g);
+    }
   } else {
     const dim3 grid(seg_start ? rows_bound : M, (N + 31) / 32, seg_start ? 1 : groups);
     if (in_is_f32) grouped_product_simt_kernel<float><<<grid, 256, 0, stream>>>(g);
