@@ -349,7 +349,8 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
   } else if (!in_is_f32 && aligned && force_simt != 1) {
     const int row_tiles = seg_start ? (rows_bound + GP_TM - 1) / GP_TM + groups : (M + GP_TM - 1) / GP_TM;
     const long wide = (long)row_tiles * ((N + 255) / 256) * (seg_start ? 1 : groups);
-    if (wide >= 2L * syn_compute_units()) {
+    // (force_simt 3: the wide waves whatever the sizes, for tests)
+    if (wide >= 8L * syn_compute_units() || force_simt == 3) {
       const dim3 grid(row_tiles, (N + 255) / 256, seg_start ? 1 : groups);
       grouped_product_mfma_kernel<4><<<grid, 256, 0, stream>>>(g);
     } else {

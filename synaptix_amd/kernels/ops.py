@@ -1109,7 +1109,8 @@ def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force
     """A linear map for each head:  out[n, h, out_offset + j] = sum_k x[n, h, k] * w[h, j, k]  [* sigmoid(gate)].
     x [N, heads, K] and w [heads, J, K] in the engine's type, out [N, heads, >= out_offset + J] in that type.
     gate: float rows (columns of a fused projection, any row stride) that hold heads * J values (one for each output,
-    gate_per_value) or `heads` values (one a head)."""
+    gate_per_value) or `heads` values (one a head).  force_simt (tests): 0 the kernel that the sizes call for, 1 plain
+    FMA, 2 and 3 the matrix cores with operands straight from memory, 16 and 64 outputs a wave."""
     _need(x, "heads_product.x", (_BF16, _F32), (None, None, None))
     N, Hn, K = x.shape
     _need(w, "heads_product.w", x.dtype, (Hn, None, K))
@@ -1168,7 +1169,7 @@ def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False,
     """out[o_rows[r]] = epilogue(x[a_rows[r]] . w[e]^T) for the places r of each expert e's segment.  x [*, K] in the
     engine's type, w [E, J, K] in that type, out [*, J] in that type or float; the index lists come from route_sort and
     must stay inside x and out (the caller sees to that: they are on the device).  Epilogue: the exact GELU, then the
-    row's weight, each if asked for."""
+    row's weight, each if asked for.  force_simt: as in heads_product."""
     _need(x, "experts_product.x", (_BF16, _F32), (None, None))
     K = x.shape[1]
     _need(w, "experts_product.w", x.dtype, (None, None, K))

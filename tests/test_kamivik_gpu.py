@@ -87,7 +87,7 @@ def test_a_linear_map_for_each_head(N, H, K, J, dtype):
     ops.heads_product(dev(x, dtype), dev(w, dtype), out, gate=G[:, 1:1 + H], gate_per_value=False)
     assert float((out.cpu().double() - plain * torch.sigmoid(gate[:, 1:1 + H])[:, :, None]).abs().max()) < tol
     if dtype == torch.bfloat16:           # all kernels give the sums of the same products
-        for force in (1, 2):              # plain FMA; the matrix cores without LDS (where K allows, else FMA again)
+        for force in (1, 2, 3):           # plain FMA; the matrix cores without LDS (where K allows, else FMA again)
             other = torch.empty_like(out)
             ops.heads_product(dev(x, dtype), dev(w, dtype), other, gate=G[:, 1:1 + H], gate_per_value=False, force_simt=force)
             assert float((other.float() - out.float()).abs().max()) < tol
@@ -124,7 +124,7 @@ def test_router_and_experts(N, W, F, E, top, dtype):
     for t in range(N):
         for e, a in zip(want_ids[t].tolist(), want_w[t]):
             want[t] += a * (downs[e] @ P.gelu(ups[e] @ h[t]))
-    for force in (0, 1, 2):
+    for force in (0, 1, 2, 3):      # by size; plain FMA; the matrix cores without LDS, 16 and 64 outputs a wave
         mid = torch.empty((N * top, F), dtype=dtype, device=DEV)
         ops.experts_product(dev(h, dtype), dev(ups, dtype), mid, seg, tok_of, pair_of, gelu=True, force_simt=force)
         y = torch.empty((top, N, W), dtype=torch.float32, device=DEV)
