@@ -14,7 +14,7 @@
 // tokens alike.
 #include "common.h"
 
-#define AW_MAX_DIM 256
+#define AW_MAX_DIM 640      // (instantiations for head sizes up to 256 and up to 640)
 
 struct WindowTerms {
   const float* slopes;   // [heads] or nullptr
@@ -125,16 +125,17 @@ template <> __device__ __forceinline__ void load8<float>(const float* p, float (
 // WAVES waves a (token, head): wave w takes every WAVES-th of the visible blocks of 64 keys, and the waves' partial
 // results (maximum, sum, weighted values) are merged through LDS at the end.  One wave is enough where a step has many
 // tokens; single tokens over a long window get eight.
-template <typename T, int WAVES>
+// MAXD: the largest head size that the registers and LDS of this instantiation hold (a multiple of 64).
+template <typename T, int WAVES, int MAXD>
 __global__ void __launch_bounds__(WAVES * SYN_WAVE)
 window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                         const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                         const int* __restrict__ tok_pos, const float* __restrict__ gate, int gate_stride,
                         const float* __restrict__ gate_bias, T* __restrict__ out, float scale, int nh, int nkv, int dim,
                         int vdim, WindowTerms terms) {
-  __shared__ float qs[AW_MAX_DIM];
+  __shared__ float qs[MAXD];
   __shared__ float ps[WAVES][SYN_PAGE];
-  __shared__ float part_o[WAVES][AW_MAX_DIM];
+  __shared__ float part_o[WAVES][MAXD];
   __shared__ float part_ml[WAVES][2];
   const int tok = blockIdx.x, head = blockIdx.y;
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
@@ -154,7 +155,7 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
   // the sink is a key of score 0 without a value: the first wave's running maximum and sum start from it
   const bool sink_here = terms.sink_one && wave == 0;
   float m = sink_here ? 0.f : -INFINITY, l = sink_here ? 1.f : 0.f;
-  float o[AW_MAX_DIM / SYN_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  float o[MAXD / SYN_WAVE] = {};
   for (int idx = wave; idx < n_blocks; idx += WAVES) {
     const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
     const int page = page_table[(size_t)seq * table_stride + kb];
@@ -192,7 +193,7 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i) {
+    for (int i = 0; i < MAXD / SYN_WAVE; ++i) {
       const int d = lane + i * SYN_WAVE;
       if (d < vdim) {
         const T* vr = v_pages + vbase + (size_t)d * SYN_PAGE;
@@ -214,7 +215,7 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     // merge in the waves' order: the largest maximum, every wave's sum and values scaled to it
     if (lane == 0) part_ml[wave][0] = m, part_ml[wave][1] = l;
 #pragma unroll
-    for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i)
+    for (int i = 0; i < MAXD / SYN_WAVE; ++i)
       if (lane + i * SYN_WAVE < vdim) part_o[wave][lane + i * SYN_WAVE] = o[i];
     __syncthreads();
     if (wave != 0) return;
@@ -222,19 +223,19 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, part_ml[w][0]);
     l = 0.f;
 #pragma unroll
-    for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i) o[i] = 0.f;
+    for (int i = 0; i < MAXD / SYN_WAVE; ++i) o[i] = 0.f;
     for (int w = 0; w < WAVES; ++w) {
       const float f = part_ml[w][0] == -INFINITY ? 0.f : expf(part_ml[w][0] - mm);
       l += f * part_ml[w][1];
 #pragma unroll
-      for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i)
+      for (int i = 0; i < MAXD / SYN_WAVE; ++i)
         if (lane + i * SYN_WAVE < vdim) o[i] += f * part_o[w][lane + i * SYN_WAVE];
     }
   }
   T* orow = out + ((size_t)tok * nh + head) * vdim;
   const float* g = gate ? gate + (size_t)tok * gate_stride + (size_t)head * vdim : nullptr;
 #pragma unroll
-  for (int i = 0; i < AW_MAX_DIM / SYN_WAVE; ++i) {
+  for (int i = 0; i < MAXD / SYN_WAVE; ++i) {
     const int d = lane + i * SYN_WAVE;
     if (d < vdim) {
       float v = o[i] / l;
@@ -266,17 +267,20 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
   const dim3 grid(n_tokens, nh);
   // few (token, head) pairs (single tokens of a few sequences): eight waves share each pair's keys
   const bool many_waves = (long)n_tokens * nh < 8L * syn_compute_units();
-#define SYN_AW(T, W)                                                                                                  \
-  window_attention_kernel<T, W><<<grid, W * SYN_WAVE, 0, stream>>>((const T*)q, (const T*)k_pages, (const T*)v_pages,   \
-                                                                   page_table, table_stride, tok_seq, tok_pos, gate,   \
-                                                                   gate_stride, gate_bias, (T*)out, scale, nh, nkv, dim, \
-                                                                   vdim, terms)
+  const bool large = dim > 256 || vdim > 256;
+#define SYN_AW2(T, W, D)                                                                                              \
+  window_attention_kernel<T, W, D><<<grid, W * SYN_WAVE, 0, stream>>>((const T*)q, (const T*)k_pages, (const T*)v_pages, \
+                                                                      page_table, table_stride, tok_seq, tok_pos, gate, \
+                                                                      gate_stride, gate_bias, (T*)out, scale, nh, nkv,  \
+                                                                      dim, vdim, terms)
+#define SYN_AW(T, W) do { if (large) SYN_AW2(T, W, 640); else SYN_AW2(T, W, 256); } while (0)
   if (is_f32) {
     if (many_waves) SYN_AW(float, 8); else SYN_AW(float, 1);
   } else {
     if (many_waves) SYN_AW(bf16, 8); else SYN_AW(bf16, 1);
   }
 #undef SYN_AW
+#undef SYN_AW2
   SYN_LAUNCH_CHECK("window_attention");
   return 0;
 }

@@ -795,7 +795,7 @@ def streams_start(x, X):
 
 # ----------------------------------------------------------------------------- attention with terms, a kept window, a sink
 
-WINDOW_ATTENTION_MAX_DIM = 256
+WINDOW_ATTENTION_MAX_DIM = 640
 
 
 def _check_window_pages(k_pages, v_pages, dtype, nkv, dim, vdim, name):

@@ -188,6 +188,26 @@ def test_latent_attention_sees_exactly_its_keys(window, dtype):
         assert float((one.cpu().double().view(H, C) - want[t]).abs().max()) < tol, f"query {t} alone"
 
 
+def test_latent_attention_over_long_rows_in_float32():
+    """Rows of 320 + 40 values through the plain kernel (its instantiation for head sizes above 256): random rows, the
+    queries long enough that the softmax is peaked; all queries at once and one alone."""
+    from synaptix_amd.kernels import ops
+    T, H, C, B, window = 150, 2, 320, 40, 65
+    g = torch.Generator().manual_seed(9)
+    rows = torch.randn(T, C + B, generator=g, dtype=P.F64)
+    q = torch.randn(T, H, C + B, generator=g, dtype=P.F64) * 0.5
+    want = P.shared_row_attention(q, rows, C, 0.3, window)
+    kp, vp, table = paged_rows(rows, C, torch.float32, shuffle_seed=3)
+    tok_seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    tok_pos = torch.arange(T, dtype=torch.int32, device=DEV)
+    out = torch.empty((T, H * C), dtype=torch.float32, device=DEV)
+    ops.latent_attention(dev(q.reshape(T, -1)), kp, vp, table, tok_seq, tok_pos, out, 0.3, H, C, B, window=window)
+    assert float((out.cpu().double().view(T, H, C) - want).abs().max()) < 5e-5
+    one = torch.empty((1, H * C), dtype=torch.float32, device=DEV)
+    ops.latent_attention(dev(q[140].reshape(1, -1)), kp, vp, table, tok_seq[:1], tok_pos[140:141], one, 0.3, H, C, B, window=window)
+    assert float((one.cpu().double().view(H, C) - want[140]).abs().max()) < 5e-5
+
+
 @pytest.mark.parametrize("H,C,B", [(3, 16, 16), (16, 32, 16), (5, 48, 0), (2, 144, 48), (20, 256, 64), (4, 512, 64)])
 @pytest.mark.parametrize("window", [0, 1, 64, 65, 130])
 def test_latent_attention_in_tiles_on_the_matrix_cores(window, H, C, B):
