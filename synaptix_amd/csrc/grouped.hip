@@ -34,7 +34,14 @@ struct GroupedArgs {
   int gate_col;
   int act;                  // 0: none, 1: exact GELU
   int M, N, K, groups;
+  int w_packed;             // W[group] lies in the order of the fragments: [N / 16][K / 32][64 lanes][8] with
+                            // lane = 16 (k % 32 / 8) + n % 16 (bf16, N a multiple of 16, K of 32); 0: plain rows
 };
+
+// element (n, k) of a matrix in fragment order, K32 = K / 32
+__device__ __forceinline__ size_t packed_at(int n, int k, int K32) {
+  return ((size_t)(n >> 4) * K32 + (k >> 5)) * 512 + (((k & 31) >> 3) << 7) + ((n & 15) << 3) + (k & 7);
+}
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
 
@@ -80,7 +87,8 @@ __global__ void __launch_bounds__(256) grouped_product_simt_kernel(GroupedArgs g
     const float x = to_f32<T>(a[k]);
 #pragma unroll
     for (int c = 0; c < 8; ++c)
-      if (n0 + c < g.N) acc[c] = fmaf(x, to_f32<T>(w[(size_t)(n0 + c) * g.ldw + k]), acc[c]);
+      if (n0 + c < g.N)
+        acc[c] = fmaf(x, to_f32<T>(w[g.w_packed ? packed_at(n0 + c, k, g.K / 32) : (size_t)(n0 + c) * g.ldw + k]), acc[c]);
   }
 #pragma unroll
   for (int c = 0; c < 8; ++c) {
@@ -136,8 +144,11 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
   for (int nb = 0; nb < NB; ++nb) {
     const int n = n0 + nb * 16 + i;
     w_ok[nb] = n < g.N;
-    wrow[nb] = W + (size_t)(w_ok[nb] ? n : 0) * g.ldw + q * 8;
+    // (in fragment order a wave's load of a k-step is 1 KB of consecutive bytes, and the next k-step lies 1 KB on)
+    wrow[nb] = g.w_packed ? W + (size_t)((w_ok[nb] ? n : 0) >> 4) * (g.K / 32) * 512 + lane * 8
+                          : W + (size_t)(w_ok[nb] ? n : 0) * g.ldw + q * 8;
   }
+  const int w_step = g.w_packed ? 512 : 32;          // elements from one k-step of 32 to the next
   f32x4 acc[2][NB];
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb)
@@ -155,7 +166,7 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) xa[u][mb] = *(const bf16x8*)(arow[mb] + k0 + 32 * u);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xw[u][nb] = __builtin_nontemporal_load((const bf16x8*)(wrow[nb] + k0 + 32 * u));
+      for (int nb = 0; nb < NB; ++nb) xw[u][nb] = __builtin_nontemporal_load((const bf16x8*)(wrow[nb] + (size_t)(k0 / 32 + u) * w_step));
     }
 #pragma unroll
     for (int u = 0; u < AHEAD; ++u) {
@@ -175,7 +186,7 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) xa[mb] = a_ok[mb] ? *(const bf16x8*)(arow[mb] + k0) : zero;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) xw[nb] = w_ok[nb] ? *(const bf16x8*)(wrow[nb] + k0) : zero;
+    for (int nb = 0; nb < NB; ++nb) xw[nb] = w_ok[nb] ? *(const bf16x8*)(wrow[nb] + (size_t)(k0 / 32) * w_step) : zero;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -251,8 +262,11 @@ __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs 
   for (int i = 0; i < WL; ++i) {
     const int n = n0 + lrow + RPP * i;
     win[i] = n < g.N;
-    wg[i] = W + (size_t)(win[i] ? n : 0) * g.ldw + lchunk;
+    const int nn = win[i] ? n : 0;
+    wg[i] = g.w_packed ? W + (size_t)(nn >> 4) * (g.K / 32) * 512 + ((nn & 15) << 3) + ((lchunk >> 5) << 9) + (((lchunk & 31) >> 3) << 7)
+                       : W + (size_t)nn * g.ldw + lchunk;
   }
+  const int w_tile = g.w_packed ? (GT_BK / 32) * 512 : GT_BK;      // elements from one k-tile to the next
   f32x16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -269,7 +283,7 @@ __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs 
 #pragma unroll
     for (int i = 0; i < XL; ++i) rx[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + k) : zero;
 #pragma unroll
-    for (int i = 0; i < WL; ++i) rw[i] = (kin && win[i]) ? *(const bf16x8*)(wg[i] + k) : zero;
+    for (int i = 0; i < WL; ++i) rw[i] = (kin && win[i]) ? *(const bf16x8*)(wg[i] + (size_t)kt * w_tile) : zero;
   };
   auto stash = [&](int buf) {
     bf16* xs = smem + buf * (GT_BM + GT_BN) * GT_LD;
@@ -320,15 +334,17 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
                                    long ldo, long o_group, int in_is_f32, int out_is_f32, const int* seg_start,
                                    const int* a_rows, const int* o_rows, const float* row_weight, const float* gate,
                                    long gate_ld, long gate_group, int gate_col, int act, int M, int N, int K, int groups,
-                                   int rows_bound, int force_simt, hipStream_t stream) {
+                                   int rows_bound, int force_simt, int w_packed, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0 && groups > 0, "grouped_product: empty input (%d rows, %d x %d, %d groups)", M, N, K, groups);
   SYN_CHECK(act == 0 || act == 1, "grouped_product: unknown activation code %d", act);
   SYN_CHECK(seg_start != nullptr || (a_rows == nullptr && o_rows == nullptr && row_weight == nullptr),
             "grouped_product: index lists and row weights come with segments");
   SYN_CHECK(seg_start == nullptr || rows_bound > 0, "grouped_product: segments over %d rows", rows_bound);
   SYN_CHECK(seg_start == nullptr || gate == nullptr, "grouped_product: a gate is read by row and group, not through segments");
+  SYN_CHECK(!w_packed || (!in_is_f32 && N % 16 == 0 && K % 32 == 0),
+            "grouped_product: matrices in fragment order are bf16 of %d x %d (multiples of 16 and 32)?", N, K);
   const GroupedArgs g = {a, lda, a_group, w, w_group, ldw, out, ldo, o_group, out_is_f32, seg_start, a_rows, o_rows,
-                         row_weight, gate, gate_ld, gate_group, gate_col, act, M, N, K, groups};
+                         row_weight, gate, gate_ld, gate_group, gate_col, act, M, N, K, groups, w_packed};
   const bool aligned = K % 32 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ldw % 8 == 0 && w_group % 8 == 0 &&
                        (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
   // many rows a group (on average, where the host does not know the segments): the tiles through LDS

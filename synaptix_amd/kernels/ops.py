@@ -1097,12 +1097,12 @@ def add_scaled_rmsnorm(resid, terms, gain, eps, out, rows=None):
 
 def _grouped(name, a, lda, a_group, w, w_group, ldw, out, ldo, o_group, M, N, K, groups, seg=None, a_rows=None,
              o_rows=None, row_weight=None, gate=None, gate_ld=0, gate_group=0, gate_col=0, act=0, rows_bound=0,
-             force_simt=False):
+             force_simt=False, w_packed=False):
     L = ctypes.c_long
     _call(load_library("core"), "syn_grouped_product", _ptr(a), L(lda), L(a_group), _ptr(w), L(w_group), L(ldw), _ptr(out),
           L(ldo), L(o_group), _is_f32(a), _is_f32(out), _ptr(seg), _ptr(a_rows), _ptr(o_rows), _ptr(row_weight), _ptr(gate),
           L(gate_ld), L(gate_group), int(gate_col), int(act), int(M), int(N), int(K), int(groups), int(rows_bound),
-          int(force_simt), _stream())
+          int(force_simt), int(bool(w_packed)), _stream())
 
 
 def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force_simt=False):
@@ -1165,15 +1165,31 @@ def route_sort(ids, weights, n_experts):
     return seg, lists[0], lists[1], lists[2], weight_of
 
 
+def pack_expert_weights(w):
+    """Matrices [E, J, K] in the order of the MFMA fragments, each as pack_weight lays it out: [E, J / 16, K / 32, 64, 8]
+    (a wave's load of a k-step is then 1 KB of consecutive bytes); None if the type or the sizes do not allow it."""
+    if w.dtype != _BF16 or w.dim() != 3 or w.shape[1] % 16 or w.shape[2] % 32:
+        return None
+    E, J, K = w.shape
+    return w.view(E, J // 16, 16, K // 32, 4, 8).permute(0, 1, 3, 4, 2, 5).reshape(E, J // 16, K // 32, 64, 8).contiguous()
+
+
 def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False, force_simt=False):
     """out[o_rows[r]] = epilogue(x[a_rows[r]] . w[e]^T) for the places r of each expert e's segment.  x [*, K] in the
-    engine's type, w [E, J, K] in that type, out [*, J] in that type or float; the index lists come from route_sort and
+    engine's type, w [E, J, K] in that type (or bf16 in fragment order, pack_expert_weights: five dimensions), out
+    [*, J] in that type or float; the index lists come from route_sort and
     must stay inside x and out (the caller sees to that: they are on the device).  Epilogue: the exact GELU, then the
     row's weight, each if asked for.  force_simt: as in heads_product."""
     _need(x, "experts_product.x", (_BF16, _F32), (None, None))
     K = x.shape[1]
-    _need(w, "experts_product.w", x.dtype, (None, None, K))
-    E, J = w.shape[0], w.shape[1]
+    packed = isinstance(w, torch.Tensor) and w.dim() == 5
+    if packed:
+        _need(x, "experts_product.x", _BF16, (None, None))
+        _need(w, "experts_product.w", _BF16, (None, None, K // 32 if K % 32 == 0 else -1, 64, 8))
+        E, J = w.shape[0], w.shape[1] * 16
+    else:
+        _need(w, "experts_product.w", x.dtype, (None, None, K))
+        E, J = w.shape[0], w.shape[1]
     _need(out, "experts_product.out", (x.dtype, _F32), (None, J))
     _need(seg, "experts_product.seg", _I32, (E + 1,))
     _need(a_rows, "experts_product.a_rows", _I32, (None,))
@@ -1182,7 +1198,7 @@ def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False,
     if row_weight is not None:
         _need(row_weight, "experts_product.row_weight", _F32, (P,))
     _grouped("experts_product", x, K, 0, w, J * K, K, out, J, 0, P, J, K, E, seg=seg, a_rows=a_rows, o_rows=o_rows,
-             row_weight=row_weight, act=1 if gelu else 0, rows_bound=P, force_simt=force_simt)
+             row_weight=row_weight, act=1 if gelu else 0, rows_bound=P, force_simt=force_simt, w_packed=packed)
 
 
 # ----------------------------------------------------------------------------- latent attention: intake

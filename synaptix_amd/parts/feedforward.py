@@ -110,8 +110,14 @@ class RoutedExperts(FeedForward):
 
     def load(self, get):
         p, (up, down, router, bias) = self.prefix, self.names
-        self.w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
-        self.w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
+        # every expert's matrices kept once: in fragment order where type and sizes allow, else in plain rows
+        w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
+        packed = ops.pack_expert_weights(w_up)
+        self.w_up = w_up if packed is None else packed
+        del w_up, packed
+        w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
+        packed = ops.pack_expert_weights(w_down)
+        self.w_down = w_down if packed is None else packed
         self.w_router = Matrix(get(p + router))
         self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
 

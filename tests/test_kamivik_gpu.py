@@ -124,13 +124,18 @@ def test_router_and_experts(N, W, F, E, top, dtype):
     for t in range(N):
         for e, a in zip(want_ids[t].tolist(), want_w[t]):
             want[t] += a * (downs[e] @ P.gelu(ups[e] @ h[t]))
-    for force in (0, 1, 2, 3):      # by size; plain FMA; the matrix cores without LDS, 16 and 64 outputs a wave
-        mid = torch.empty((N * top, F), dtype=dtype, device=DEV)
-        ops.experts_product(dev(h, dtype), dev(ups, dtype), mid, seg, tok_of, pair_of, gelu=True, force_simt=force)
-        y = torch.empty((top, N, W), dtype=torch.float32, device=DEV)
-        ops.experts_product(mid, dev(downs, dtype), y.view(top * N, W), seg, pair_of, part_of, row_weight=weight_of,
-                            force_simt=force)
-        assert float((y.sum(0).cpu().double() - want).abs().max()) < (5e-5 if dtype == torch.float32 else 5e-2)
+    w_up, w_down = dev(ups, dtype), dev(downs, dtype)
+    kept = [(w_up, w_down)]
+    if dtype == torch.bfloat16 and ops.pack_expert_weights(w_up) is not None and ops.pack_expert_weights(w_down) is not None:
+        kept.append((ops.pack_expert_weights(w_up), ops.pack_expert_weights(w_down)))      # in fragment order
+    for w_up, w_down in kept:
+        for force in (0, 1, 2, 3):      # by size; plain FMA; the matrix cores without LDS, 16 and 64 outputs a wave
+            mid = torch.empty((N * top, F), dtype=dtype, device=DEV)
+            ops.experts_product(dev(h, dtype), w_up, mid, seg, tok_of, pair_of, gelu=True, force_simt=force)
+            y = torch.empty((top, N, W), dtype=torch.float32, device=DEV)
+            ops.experts_product(mid, w_down, y.view(top * N, W), seg, pair_of, part_of, row_weight=weight_of,
+                                force_simt=force)
+            assert float((y.sum(0).cpu().double() - want).abs().max()) < (5e-5 if dtype == torch.float32 else 5e-2)
 
 
 def paged_rows(rows, n_values, dtype, shuffle_seed=0):
