@@ -91,9 +91,9 @@ class LogDistanceBias(Position):
 
 class RotaryInterleaved(Position):
     """A rotation of the pairs (2i, 2i + 1), i < dims / 2, of a vector's first `dims` values by the angle
-    position * base^(-2i / dims); what lies behind `dims` passes unchanged.  The pair (u, v) becomes
-    (u cos a - v sin a, v cos a + u sin a).  Tables [capacity, dims / 2] are made on the host with 64-bit angles and
-    kept in 32-bit, once for all parts with the same constants."""
+    t_i = position * base^(-2i / dims), as a complex multiplication (x_2i + j x_2i+1) e^(j t_i); what lies behind `dims`
+    passes unchanged.  Tables [capacity, dims / 2] are made on the host with 64-bit angles and kept in 32-bit, once for
+    all parts with the same constants."""
     capturable = True
     _shared: dict = {}
 
