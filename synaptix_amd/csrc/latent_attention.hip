@@ -18,8 +18,8 @@
 // and weights are 32-bit; a weight meets V as two bf16 numbers (the weight rounded, and what the rounding left), so
 // it counts with 16 bits of mantissa although the product runs in bf16; sums are 32-bit.
 // A tile's pages may be cut into splits (grid y) whose partial results a second kernel merges, and (SHARE) the four
-// waves of a workgroup may take one tile's pages in turns and merge through LDS: single tokens over long sequences
-// then fill the chip.
+// waves of a workgroup may work on one tile together: single tokens over long sequences then fill the chip, and no
+// wave walks a page alone.
 #include "common.h"
 
 #define LA_ROWS 16
@@ -35,20 +35,6 @@ __device__ __forceinline__ f32x4 la_mfma(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// the sequence and the tile inside it of global tile t; false: beyond the last tile
-__device__ __forceinline__ bool la_find_tile(int t, const int* seq_start, int n_seqs, int nh, int& seq, int& tile,
-                                             int& start, int& rows) {
-  for (int b = 0; b < n_seqs; ++b) {
-    const int s0 = seq_start[b], n = (seq_start[b + 1] - s0) * nh, tiles = (n + LA_ROWS - 1) / LA_ROWS;
-    if (t < tiles) {
-      seq = b, tile = t, start = s0, rows = n;
-      return true;
-    }
-    t -= tiles;
-  }
-  return false;
-}
-
 // Where value d of the token in slot `slot` of a page lies in a bf16 value page of latent attention: fragment (d / 16,
 // slot / 32), lane 16 g + d % 16, element e, with the 32 slots of a half in the order in which two tiles of scores
 // leave them in a lane: e < 4: slot 4 g + e; e >= 4: slot 16 + 4 g + (e - 4).
@@ -57,16 +43,34 @@ __host__ __device__ __forceinline__ int la_v_offset(int d, int slot) {
   return ((((d >> 4) * 2 + half) * 64 + g * 16 + (d & 15)) << 3) + e;
 }
 
-// the sequence and the unit inside it of global unit t, a unit being `unit_rows` consecutive (token, head) rows
+// the sequence and the unit inside it of global unit t, a unit being `unit_rows` consecutive (token, head) rows.
+// Every wave searches for itself, 64 sequences at a time: a lane a sequence, a prefix sum of their units across the
+// lanes, the first lane whose sum passes t (one trip to memory for 64 sequences, not one for each).  t is the same in
+// all lanes of the wave.
 __device__ __forceinline__ bool la_find_unit(int t, int unit_rows, const int* seq_start, int n_seqs, int nh, int& seq,
                                              int& unit, int& start, int& rows) {
-  for (int b = 0; b < n_seqs; ++b) {
-    const int s0 = seq_start[b], n = (seq_start[b + 1] - s0) * nh, units = (n + unit_rows - 1) / unit_rows;
-    if (t < units) {
-      seq = b, unit = t, start = s0, rows = n;
+  const int lane = threadIdx.x % SYN_WAVE;
+  for (int b0 = 0; b0 < n_seqs; b0 += SYN_WAVE) {
+    const int b = b0 + lane;
+    const int s0 = b < n_seqs ? seq_start[b] : 0;
+    const int n = b < n_seqs ? (seq_start[b + 1] - s0) * nh : 0;
+    const int units = (n + unit_rows - 1) / unit_rows;
+    int upto = units;                                    // units of the sequences b0 .. b
+#pragma unroll
+    for (int off = 1; off < SYN_WAVE; off <<= 1) {
+      const int other = __shfl_up(upto, off, SYN_WAVE);
+      if (lane >= off) upto += other;
+    }
+    const unsigned long long found = __ballot(t < upto);
+    if (found) {
+      const int at = __ffsll((long long)found) - 1;
+      seq = b0 + at;
+      unit = t - (__shfl(upto, at, SYN_WAVE) - __shfl(units, at, SYN_WAVE));
+      start = __shfl(s0, at, SYN_WAVE);
+      rows = __shfl(n, at, SYN_WAVE);
       return true;
     }
-    t -= units;
+    t -= __shfl(upto, SYN_WAVE - 1, SYN_WAVE);
   }
   return false;
 }
@@ -76,7 +80,7 @@ __device__ __forceinline__ bool la_find_unit(int t, int unit_rows, const int* se
 // SHARE false (prompts): a workgroup takes four consecutive tiles of one sequence, a wave each, and walks the pages
 // that any of them sees: a page's keys and values go through LDS once for the four (rows of keys padded by 16 bytes
 // against bank conflicts; dynamic LDS: 64 (R + 8) + 64 rank bf16 values).  SHARE true (single tokens): a workgroup
-// takes one tile, its waves the tile's pages in turns, operands straight from memory, merged through LDS at the end.
+// takes one tile; on every page its four waves split the keys for the scores and the values for the second product.
 template <int DT, int QS, bool X32, bool SHARE>
 __global__ void __launch_bounds__(256)
 latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
@@ -110,9 +114,13 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   for (int ks = 0; ks < QS; ++ks)
     if (ks < n_qs) qf[ks] = *(const frag*)(qrow + ks * KS);
 
-  f32x4 acc[DT];
+  // SHARE: a wave holds a quarter of the value tiles (DTW of them, from dt0 on); else all of them
+  constexpr int DTW = SHARE ? DT / 4 : DT;
+  const int dt0 = SHARE ? wave * ((n_dt + 3) / 4) : 0;
+  const int dt_end = SHARE ? min(dt0 + (n_dt + 3) / 4, n_dt) : n_dt;
+  f32x4 acc[DTW];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int dt = 0; dt < DTW; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int* pages = page_table + (size_t)seq * table_stride;
 
@@ -164,7 +172,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     l = l * alpha + sum;
     m = m_new;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DTW; ++dt)
       if (dt < n_dt) acc[dt] *= alpha;
     // slots behind the sequence's end may hold anything: their weights are 0, their values are made 0 as well
     const int left = kv_len - p * SYN_PAGE;
@@ -177,7 +185,7 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         pl[e] = lo[2 * half][e], pl[4 + e] = lo[2 * half + 1][e];
       }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DTW; ++dt)
         if (dt < n_dt) {
           bf16x8 a = *(const bf16x8*)(vb + (dt * 2 + half) * 512);
           if (left < SYN_PAGE) {
@@ -194,13 +202,92 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   };
 
   if constexpr (SHARE) {
-    // this split's share of the tile's pages, a page a wave in turns, operands straight from memory
+    // This split's share of the tile's pages, one after another, the four waves on the same page: wave w multiplies
+    // the 16 keys w * 16 .. of the page with the queries, the waves exchange maxima, sums and weights through LDS (the
+    // weights already in the order of the second product's operand), and wave w then multiplies its quarter of the
+    // value tiles with all 64 weights.  Every load of a phase is asked for before the first result is needed, the
+    // values before the scores are exchanged.  What goes through LDS is kept twice, for pages in turns: two barriers
+    // a page are enough.
+    __shared__ float sh_max[2][4][LA_ROWS], sh_sum[2][4][LA_ROWS];
+    __shared__ __attribute__((aligned(16))) bf16 sh_hi[2][2][SYN_WAVE][8], sh_lo[2][2][SYN_WAVE][8];
     const int chunk = (my_hi - my_lo + n_splits) / n_splits;
     const int p0 = my_lo + split * chunk, p1 = min(p0 + chunk, my_hi + 1);
-    for (int p = p0 + wave; p < p1; p += 4) {
+    int par = 0;
+    for (int p = p0; p < p1; ++p, par ^= 1) {
       const int page = pages[p];
-      one_page(k_pages + (size_t)page * SYN_PAGE * R + (size_t)i * R + g * PIECE, R,
-               v_pages + (size_t)page * rank * SYN_PAGE + lane * 8, p);
+      const bf16* kb = k_pages + (size_t)page * SYN_PAGE * R + (size_t)(wave * 16 + i) * R + g * PIECE;
+      const bf16* vb = v_pages + (size_t)page * rank * SYN_PAGE + lane * 8;
+      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < QS; ++ks)
+        if (ks < n_qs) s = la_mfma(*(const frag*)(kb + ks * KS), qf[ks], s);
+      bf16x8 va[DTW][2];
+#pragma unroll
+      for (int j = 0; j < DTW; ++j)
+        if (dt0 + j < dt_end) {
+          va[j][0] = *(const bf16x8*)(vb + ((dt0 + j) * 2) * 512);
+          va[j][1] = *(const bf16x8*)(vb + ((dt0 + j) * 2 + 1) * 512);
+        }
+      // s[e]: key p * 64 + wave * 16 + 4 g + e against this lane's row
+      const int key0 = p * SYN_PAGE + wave * 16 + 4 * g;
+      float top = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + e;
+        const bool seen = key <= pos && (window <= 0 || pos - key < window);
+        s[e] = seen ? s[e] * scale : -INFINITY;
+        top = fmaxf(top, s[e]);
+      }
+      top = fmaxf(top, __shfl_xor(top, 16, SYN_WAVE));
+      top = fmaxf(top, __shfl_xor(top, 32, SYN_WAVE));
+      if (g == 0) sh_max[par][wave][i] = top;
+      __syncthreads();
+      float m_new = m;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) m_new = fmaxf(m_new, sh_max[par][w][i]);
+      const float base = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = expf(m - base);
+      float sum = 0.f;
+      bf16x4 hi, lo;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = expf(s[e] - base);
+        sum += w;
+        hi[e] = (bf16)w;
+        lo[e] = (bf16)(w - (float)hi[e]);
+      }
+      sum += __shfl_xor(sum, 16, SYN_WAVE);
+      sum += __shfl_xor(sum, 32, SYN_WAVE);
+      if (g == 0) sh_sum[par][wave][i] = sum;
+      // key tile `wave` is elements 4 (wave % 2) .. of the operand of half wave / 2
+      *(bf16x4*)&sh_hi[par][wave >> 1][lane][4 * (wave & 1)] = hi;
+      *(bf16x4*)&sh_lo[par][wave >> 1][lane][4 * (wave & 1)] = lo;
+      __syncthreads();
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) total += sh_sum[par][w][i];
+      l = l * alpha + total;
+      m = m_new;
+      const int left = kv_len - p * SYN_PAGE;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const bf16x8 ph = *(const bf16x8*)&sh_hi[par][half][lane][0], pl = *(const bf16x8*)&sh_lo[par][half][lane][0];
+#pragma unroll
+        for (int j = 0; j < DTW; ++j)
+          if (dt0 + j < dt_end) {
+            if (half == 0) acc[j] *= alpha;
+            bf16x8 a = va[j][half];
+            if (left < SYN_PAGE) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (32 * half + 4 * g + e >= left) a[e] = (bf16)0.f;
+                if (32 * half + 16 + 4 * g + e >= left) a[4 + e] = (bf16)0.f;
+              }
+            }
+            acc[j] = la_mfma(a, ph, acc[j]);
+            acc[j] = la_mfma(a, pl, acc[j]);
+          }
+      }
     }
   } else {
     // the pages that any of the workgroup's four tiles sees, each through LDS once
@@ -229,61 +316,33 @@ latent_attention_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     }
     if (!tile_ok) return;
   }
-  // acc[dt][e]: value dt * 16 + 4 g + e of this lane's row
-  if constexpr (SHARE) {
-    // waves 1 .. 3 hand their maximum, sum and values to wave 0 through LDS, one after another
-    __shared__ float share_ml[2 * LA_ROWS];
-    __shared__ __attribute__((aligned(16))) float share_o[LA_ROWS * 16 * DT];
-    for (int w = 1; w < 4; ++w) {
-      if (wave == w) {
-        if (g == 0) share_ml[2 * i] = m, share_ml[2 * i + 1] = l;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          if (dt < n_dt) *(f32x4*)(share_o + (i * DT + dt) * 16 + 4 * g) = acc[dt];
-      }
-      __syncthreads();
-      if (wave == 0) {
-        const float mo = share_ml[2 * i], lo_ = share_ml[2 * i + 1];
-        const float mn = fmaxf(m, mo), base = mn == -INFINITY ? 0.f : mn;
-        const float fa = expf(m - base), fb = expf(mo - base);
-        l = l * fa + lo_ * fb;
-        m = mn;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          if (dt < n_dt) {
-            const f32x4 o = *(const f32x4*)(share_o + (i * DT + dt) * 16 + 4 * g);
-            acc[dt] = acc[dt] * fa + o * fb;
-          }
-      }
-      __syncthreads();
-    }
-    if (wave != 0) return;
-  }
+  // acc[j][e]: value (dt0 + j) * 16 + 4 g + e of this lane's row
   if (n_splits == 1) {
     if (!row_ok) return;
     const float inv = 1.f / l;
     bf16* orow = out + ((size_t)(start + tok) * nh + head) * rank + 4 * g;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      if (dt < n_dt) {
+    for (int j = 0; j < DTW; ++j)
+      if (dt0 + j < dt_end) {
         bf16x4 r;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r[e] = (bf16)(acc[dt][e] * inv);
-        *(bf16x4*)(orow + dt * 16) = r;
+        for (int e = 0; e < 4; ++e) r[e] = (bf16)(acc[j][e] * inv);
+        *(bf16x4*)(orow + (dt0 + j) * 16) = r;
       }
   } else {
     // (SHARE only: blockIdx.x is the tile's number among all tiles)
     const size_t at = ((size_t)blockIdx.x * n_splits + split) * LA_ROWS + i;
-    if (g == 0) part_ml[2 * at] = m, part_ml[2 * at + 1] = l;
+    if (g == 0 && wave == 0) part_ml[2 * at] = m, part_ml[2 * at + 1] = l;
     float* prow = part_o + at * rank + 4 * g;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      if (dt < n_dt) *(f32x4*)(prow + dt * 16) = acc[dt];
+    for (int j = 0; j < DTW; ++j)
+      if (dt0 + j < dt_end) *(f32x4*)(prow + (dt0 + j) * 16) = acc[j];
   }
 }
 
 // the splits of a tile merged in their order: the largest maximum, every split's sum and values scaled to it.
-// One workgroup a (tile, row): the splits' factors once in LDS, then a thread a value.
+// One workgroup a (tile, row): the splits' maxima and sums fetched side by side, their factors in LDS, then a thread a
+// value.
 #define LA_MAX_SPLITS 1024
 __global__ void __launch_bounds__(256)
 latent_attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -293,21 +352,31 @@ latent_attention_merge_kernel(const float* __restrict__ part_o, const float* __r
   __shared__ float red[16];
   const int gt = blockIdx.x, r = blockIdx.y;
   int seq, tile, start, rows;
-  if (!la_find_tile(gt, seq_start, n_seqs, nh, seq, tile, start, rows)) return;
+  if (!la_find_unit(gt, LA_ROWS, seq_start, n_seqs, nh, seq, tile, start, rows)) return;
   const int flat = tile * LA_ROWS + r;
   if (flat >= rows) return;                 // (the whole workgroup)
   const size_t at0 = (size_t)gt * n_splits * LA_ROWS + r;
+  float top = -INFINITY;
+  for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
+    const float ms = part_ml[2 * (at0 + (size_t)s * LA_ROWS)];
+    factor[s] = ms;
+    top = fmaxf(top, ms);
+  }
+  // the largest maximum of all splits: through LDS (block_sum's barriers also publish `factor`)
+  top = wave_max(top);
+  if (threadIdx.x % SYN_WAVE == 0) red[threadIdx.x / SYN_WAVE] = top;
+  __syncthreads();
   float mm = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[2 * (at0 + (size_t)s * LA_ROWS)]);
+  for (int w = 0; w < 4; ++w) mm = fmaxf(mm, red[w]);
+  __syncthreads();
   float part = 0.f;
   for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
-    const size_t at = at0 + (size_t)s * LA_ROWS;
-    const float ms = part_ml[2 * at];
+    const float ms = factor[s];
     const float f = ms == -INFINITY ? 0.f : expf(ms - mm);
     factor[s] = f;
-    part += f * part_ml[2 * at + 1];
+    part += f * part_ml[2 * (at0 + (size_t)s * LA_ROWS) + 1];
   }
-  const float l = block_sum(part, red);     // (its barriers also publish `factor`)
+  const float l = block_sum(part, red);
   bf16* orow = out + ((size_t)(start + flat / nh) * nh + flat % nh) * rank;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float o = 0.f;

@@ -1278,9 +1278,9 @@ def _latent_tiles(n_tokens, n_heads, n_seqs, max_pages):
     if tiles >= 256:
         # (a workgroup for every four tiles of a sequence: the bound counts those)
         return (n_tokens * n_heads + 63) // 64 + n_seqs, 1, False
-    # few tiles: the four waves of a workgroup share a tile's pages, and the pages are cut further until some 1,024
-    # workgroups have work
-    return tiles, max(1, min((int(max_pages) + 3) // 4, 1024 // tiles, 1024)), True
+    # few tiles: the four waves of a workgroup work on a tile together, and its pages are cut into splits until some
+    # 1,024 workgroups have work
+    return tiles, max(1, min(int(max_pages), 1024 // tiles, 1024)), True
 
 
 def latent_attention_workspace(n_tokens, n_heads, n_seqs, rank, max_pages) -> int:
